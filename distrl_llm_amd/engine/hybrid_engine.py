@@ -25,7 +25,8 @@ import torch.nn.functional as F
 
 from ..config import EngineConfig, SamplingParams
 from ..models.hybrid import (DeltaRuleSpec, GluSpec, HybridLM,
-                             LatentAttentionSpec, SinkAttentionSpec)
+                             LatentAttentionSpec, ParallelMixerSpec,
+                             SigmoidAttentionSpec, SinkAttentionSpec)
 from ..ops import functional as OF
 from ..ops import seqmix as SM
 from ..utils.trace import trace_range
@@ -114,6 +115,7 @@ class HybridEngine:
                                     self.dtype, self.device)
         self.slots = StateSlotPool(self.spec, num_slots, self.device)
         self._decode_graphs = {}     # padded rows -> _DecodeGraph
+        self._consts = {}            # small per-unit device tensors
 
     def _derive_num_blocks(self, num_slots: int) -> int:
         bs = self.cfg.kv_block_size
@@ -309,39 +311,70 @@ class HybridEngine:
             q.context_len += len(toks)
         return logits
 
-    # ---- mixers: (layer index, specs, weights, mixer input) -> [T, width]
+    # ---- mixers: (unit key, spec, weights, mixer input, step metadata) ->
+    # [T, width]. ``proj`` carries the unit's rows of a projection the caller
+    # already made (the sides of a parallel pair share one GEMM); ``x32`` is
+    # the fp32 form of the mixer input where a block has one.
 
-    def _mix_latent(self, i, m, L, hm, meta):
+    def _const(self, key, make):
+        """Small per-unit device constants (frequency tables, slopes)."""
+        c = self._consts.get(key)
+        if c is None:
+            c = self._consts[key] = make()
+        return c
+
+    def _mix_latent(self, i, m, L, hm, meta, proj=None, x32=None):
         S, dt, T = self.spec, self.dtype, hm.shape[0]
         own = m.kv_from is None
-        proj = F.linear(hm, L.in_w)
-        cache = self.pool.layer_rows(S, i)
+        if proj is None:
+            proj = F.linear(hm, L.in_w)
+        cache = self.pool.unit_rows(i, m)
+        nq = m.q_rank if m.q_rank else m.q_size
+        if m.q_rank:
+            # queries through a normed latent
+            _, cq = SM.offset_rmsnorm(proj[:, :nq], L.q_norm_w, S.norm_eps, dt, 0.0)
+            q = F.linear(cq, L.uq)
+        else:
+            q = proj[:, :nq]
+        dkv = proj[:, nq:nq + m.cache_width] if own else None
+        gate = None
+        if m.out_gate:
+            g0 = nq + (m.cache_width if own else 0)
+            gate = proj[:, g0:g0 + m.heads]
+        freqs, mag = None, 1.0
+        if m.rope_pairs or m.rope_scaling:
+            f, mag = m.rope_table()
+            freqs = self._const(("rope", i), lambda: torch.tensor(
+                f, dtype=torch.float64).to(torch.float32).to(self.device))
         q_rot = SM.latent_prepare(
-            proj, m.heads, m.dim, m.rot_dim, m.kv_rank, own,
+            q, dkv, m.heads, m.dim, m.rot_dim, m.kv_rank,
             L.latent_norm_w if own else None, S.norm_eps, meta["positions"],
-            m.rope_base, m.rope_dims, meta["page_slot"], cache)
-        q_nope = proj[:, :m.q_size].view(T, m.heads, m.dim + m.rot_dim)
+            m.rope_base, m.rope_dims, meta["page_slot"], cache, freqs, mag,
+            m.rope_pairs)
+        q_nope = q.view(T, m.heads, m.dim + m.rot_dim)
         q_lat = torch.bmm(q_nope[..., :m.dim].transpose(0, 1), L.uk)
         o_lat = SM.latent_window_attention(
             q_lat, q_rot, cache, m.kv_rank, meta["block_tables"],
             self.pool.block_size, meta["cu"], meta["tok_seq"],
             meta["positions"], m.window, m.scale, dt,
-            tiles=meta["tiles"], max_tile=meta["max_tile"])
+            tiles=meta["tiles"], max_tile=meta["max_tile"],
+            sink=L.sink if m.sink else None, gate=gate)
         v = torch.bmm(o_lat, L.uv.transpose(1, 2))
         return F.linear(v.transpose(0, 1).reshape(T, m.heads * m.vdim), L.out_w)
 
-    def _mix_mingru(self, i, m, L, hm, meta):
-        zxg = F.linear(hm, L.in_w)
+    def _mix_mingru(self, i, m, L, hm, meta, proj=None, x32=None):
+        zxg = F.linear(hm, L.in_w) if proj is None else proj
         a = SM.mingru_scan(zxg, L.in_b, self.slots.recurrent[i], meta["cu"],
                            meta["slots"], self.dtype, meta["scan_chunks"],
                            meta["scan_cu"])
         return F.linear(a, L.out_w)
 
-    def _mix_sink_attention(self, i, m, L, hm, meta, shared):
+    def _mix_sink_attention(self, i, m, L, hm, meta, shared, proj=None):
         """``shared`` carries the first value-mixing layer's fresh values of
         this step's tokens to the later mixing layers."""
-        proj = F.linear(hm, L.in_w)
-        cache = self.pool.layer_rows(self.spec, i)
+        if proj is None:
+            proj = F.linear(hm, L.in_w)
+        cache = self.pool.unit_rows(i, m)
         v_first = shared.get(("v", m.v_first)) if m.v_first is not None else None
         q = SM.rope_kv_write(proj, m.heads, m.kv_heads, m.dim, m.vdim,
                              meta["positions"], m.rope_base, m.rope_dims,
@@ -356,41 +389,85 @@ class HybridEngine:
                               max_tile=meta["max_wide_tile"])
         return F.linear(o, L.out_w)
 
-    def _mix_delta(self, i, m, L, hm, meta):
-        proj = F.linear(hm, L.in_w)
+    def _mix_sigmoid_attention(self, i, m, L, hm, meta, proj=None, x32=None):
+        if proj is None:
+            proj = F.linear(hm, L.in_w)
+        cache = self.pool.unit_rows(i, m)
+        q = SM.qk_norm_kv_write(proj, m.heads, m.kv_heads, m.dim, m.vdim,
+                                L.q_norm_w, L.k_norm_w, self.spec.norm_eps,
+                                meta["page_slot"], cache)
+        slopes = self._const(("slopes", i), lambda: torch.tensor(
+            m.slopes(), dtype=torch.float64).to(torch.float32).to(self.device))
+        o = SM.sigmoid_attention(q, cache, m.heads, m.kv_heads, m.dim, m.vdim,
+                                 meta["block_tables"], self.pool.block_size,
+                                 meta["cu"], meta["tok_seq"], meta["positions"],
+                                 m.scale, m.window, m.keep_first, slopes,
+                                 L.pos_bias, self.dtype,
+                                 tiles=meta["wide_tiles"],
+                                 max_tile=meta["max_wide_tile"])
+        return F.linear(o, L.out_w)
+
+    def _mix_delta(self, i, m, L, hm, meta, proj=None, x32=None):
+        if proj is None:
+            proj = F.linear(hm, L.in_w)
         C = m.conv_channels
         qkv = SM.tap_conv_silu(proj[:, :C], L.conv_w, self.slots.mixer_tails[i],
                                meta["cu"], meta["tok_seq"], meta["slots"],
                                self.dtype)
-        # fp32 decay / strength inputs: a GEMM for prompt-sized steps; steps
-        # of a few tokens project them inside the op (two launches fewer)
-        if hm.shape[0] <= 256:
-            ab, own = None, dict(h=hm, ab_w=L.ab_w)
-        else:
+        gate = proj[:, C:C + (m.gate_rank or m.v_size)]
+        if m.gate_rank:
+            gate = F.linear(gate, L.gate_up)
+        # fp32 strength / decay inputs: read from the fp32 mixer input where
+        # the block has one. Per-head decays: a GEMM for prompt-sized steps,
+        # steps of a few tokens project them inside the op (two launches
+        # fewer); per-channel decays always take the GEMM.
+        if x32 is not None:
+            ab, own = F.linear(x32, L.ab_w), {}
+        elif m.decay == "channel" or hm.shape[0] > 256:
             ab, own = F.linear(hm.float(), L.ab_w), {}
-        o = SM.gated_delta_rule(qkv, proj[:, C:], ab, L.a_log, L.dt_bias,
+        else:
+            ab, own = None, dict(h=hm, ab_w=L.ab_w)
+        o = SM.gated_delta_rule(qkv, gate, ab, L.a_log, L.dt_bias,
                                 L.onorm_w, self.spec.norm_eps,
                                 self.slots.recurrent[i], meta["cu"],
                                 meta["slots"], m.heads, m.kv_heads, m.dim,
-                                m.vdim, self.dtype, **own)
+                                m.vdim, self.dtype,
+                                decay_up=(L.decay_up if m.decay == "channel"
+                                          else None),
+                                gate_sigmoid=(m.gate == "sigmoid"), **own)
         return F.linear(o, L.out_w)
 
-    def _mixer(self, i, ls, L, hm, meta, shared):
-        m = ls.mixer
+    def _mix_unit(self, key, m, W, hm, meta, shared, proj=None, x32=None):
         if isinstance(m, LatentAttentionSpec):
-            return self._mix_latent(i, m, L, hm, meta)
+            return self._mix_latent(key, m, W, hm, meta, proj, x32)
         if isinstance(m, SinkAttentionSpec):
-            return self._mix_sink_attention(i, m, L, hm, meta, shared)
+            return self._mix_sink_attention(key, m, W, hm, meta, shared, proj)
+        if isinstance(m, SigmoidAttentionSpec):
+            return self._mix_sigmoid_attention(key, m, W, hm, meta, proj, x32)
         if isinstance(m, DeltaRuleSpec):
-            return self._mix_delta(i, m, L, hm, meta)
-        return self._mix_mingru(i, m, L, hm, meta)
+            return self._mix_delta(key, m, W, hm, meta, proj, x32)
+        return self._mix_mingru(key, m, W, hm, meta, proj, x32)
+
+    def _mixer(self, i, ls, L, hm, meta, shared, x32=None):
+        """-> (output, second output or None, their scales)."""
+        m = ls.mixer
+        if isinstance(m, ParallelMixerSpec):
+            proj = F.linear(hm, L.in_w)
+            nl = m.left.in_size
+            left = self._mix_unit((i, 0), m.left, L.left, hm, meta, shared,
+                                  proj[:, :nl], x32)
+            right = self._mix_unit((i, 1), m.right, L.right, hm, meta, shared,
+                                   proj[:, nl:], x32)
+            return left, right, (m.left_scale, m.right_scale)
+        return self._mix_unit(i, m, L, hm, meta, shared, None, x32), None, (1.0, 1.0)
 
     # ---- feed-forwards: -> (main output, second addend or None)
 
     def _ff(self, f, L, hb):
         if isinstance(f, GluSpec):
-            return F.linear(SM.capped_glu(F.linear(hb, L.gu_w), f.limit),
-                            L.down_w), None
+            gu = F.linear(hb, L.gu_w)
+            act = SM.silu_glu(gu) if f.act == "silu" else SM.capped_glu(gu, f.limit)
+            return F.linear(act, L.down_w), None
         if f.routing == "all":
             idx, wts = SM.moe_route_all(hb, L.router_w, L.correction, f.top,
                                         f.scale)
@@ -408,13 +485,17 @@ class HybridEngine:
         S, M, dt = self.spec, self.model, self.dtype
         if S.block == "sandwich":
             x = self._layers_sandwich(tokens, meta, capture)
+        elif S.block == "post_norm":
+            x = self._layers_post_norm(tokens, meta, capture)
         else:
             x = self._layers_parallel_gated(tokens, meta, capture)
         if want_rows.numel() == 0:
             return torch.empty(0, S.vocab_size, dtype=torch.float32,
                                device=x.device)
-        _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, S.norm_eps, dt)
-        return F.linear(hb, M.head).float()
+        _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, S.norm_eps, dt,
+                                  S.norm_offset)
+        logits = F.linear(hb, M.head).float()
+        return logits * S.logit_scale if S.logit_scale != 1.0 else logits
 
     def _layers_parallel_gated(self, tokens, meta, capture):
         """One norm per layer feeds the mixer (through the block's short
@@ -434,7 +515,7 @@ class HybridEngine:
             else:
                 hm = hb
             gates = F.linear(hb, L.gate_w)
-            y = self._mixer(i, ls, L, hm, meta, shared)
+            y = self._mixer(i, ls, L, hm, meta, shared)[0]
             f = None
             if ls.mlp is not None:
                 f, f2 = self._ff(ls.mlp, L, hb)
@@ -462,7 +543,7 @@ class HybridEngine:
         _, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt)
         last = S.num_layers - 1
         for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
-            y = self._mixer(i, ls, L, hb, meta, shared)
+            y = self._mixer(i, ls, L, hb, meta, shared)[0]
             nxt = M.layers[i + 1].norm_w if i < last else None
             hb = SM.sandwich_residual_norm(
                 x, y, None, L.post_w,
@@ -470,6 +551,32 @@ class HybridEngine:
             if ls.mlp is not None:
                 f, f2 = self._ff(ls.mlp, L, hb)
                 hb = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, nxt, eps, dt)
+            if capture is not None:
+                capture.append(x.clone())
+        return x
+
+    def _layers_post_norm(self, tokens, meta, capture):
+        """x += norm(mixer(x)), then x += norm(ff(x)): the sublayers read
+        the residual itself (in the model dtype for the matrix products, in
+        fp32 where a recurrence's inputs are formed) and only their output
+        is normed. The closing norm, the residual sum and the copy of the
+        new residual in the model dtype are one kernel; a parallel pair's
+        two outputs are scaled and summed there as well."""
+        S, M, dt = self.spec, self.model, self.dtype
+        eps, off = S.norm_eps, S.norm_offset
+        shared = {}
+        x = M.embed[tokens].float()
+        if S.embed_scale != 1.0:
+            x = x * S.embed_scale
+        hb = x.to(dt)
+        for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
+            y, y2, (a, b) = self._mixer(i, ls, L, hb, meta, shared, x32=x)
+            hb = SM.sandwich_residual_norm(x, y, y2, L.post_w, None, eps, dt,
+                                           off, a, b, cast_next=True)
+            if ls.mlp is not None:
+                f, f2 = self._ff(ls.mlp, L, hb)
+                hb = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, None, eps,
+                                               dt, off, cast_next=True)
             if capture is not None:
                 capture.append(x.clone())
         return x

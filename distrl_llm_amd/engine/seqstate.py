@@ -9,6 +9,8 @@ come and go:
   values of all kv heads]`` for grouped-query attention. Block ids come
   from the same refcounting :class:`BlockAllocator` as the dense models'
   K/V pool, so a forked candidate shares its prompt's full pages.
+  Tensors are keyed by mixer unit: the layer index, or (layer, side) for
+  the two sides of a parallel pair.
 * :class:`StateSlotPool` — fixed-size fp32 state per live sequence: the
   last ``taps - 1`` inputs of every short convolution (the block's own, or
   a delta-rule layer's over its q/k/v channels) and the state of every
@@ -24,7 +26,8 @@ from typing import Dict, List
 import torch
 
 from ..models.hybrid import (DeltaRuleSpec, HybridSpec, LatentAttentionSpec,
-                             MinGRUSpec, SinkAttentionSpec)
+                             MinGRUSpec, SigmoidAttentionSpec,
+                             SinkAttentionSpec, mixer_units)
 from .kvcache import BlockAllocator
 
 
@@ -37,23 +40,24 @@ class LatentCachePool:
         # one page past the allocator's range that no sequence ever owns:
         # padding rows of a captured decode step write there
         self.scratch_block = num_blocks
-        # layer index -> [(num_blocks + 1) * block_size, kv_rank + rot_dim]
-        self.rows: Dict[int, torch.Tensor] = {}
-        for i, ls in enumerate(spec.layers):
-            m = ls.mixer
+        # mixer unit -> [(num_blocks + 1) * block_size, cache row width]
+        self.rows: Dict[object, torch.Tensor] = {}
+        for i, m in mixer_units(spec):
             if self._owns_rows(m):
                 self.rows[i] = torch.zeros((num_blocks + 1) * block_size, m.cache_width,
                                            dtype=dtype, device=device)
 
     @staticmethod
     def _owns_rows(m) -> bool:
-        return (isinstance(m, SinkAttentionSpec)
+        return (isinstance(m, (SinkAttentionSpec, SigmoidAttentionSpec))
                 or (isinstance(m, LatentAttentionSpec) and m.kv_from is None))
 
     def layer_rows(self, spec: HybridSpec, layer: int) -> torch.Tensor:
-        m = spec.layers[layer].mixer
+        return self.unit_rows(layer, spec.layers[layer].mixer)
+
+    def unit_rows(self, key, m) -> torch.Tensor:
         src = getattr(m, "kv_from", None)
-        return self.rows[layer if src is None else src]
+        return self.rows[key if src is None else src]
 
     @staticmethod
     def blocks_for(num_tokens: int, block_size: int) -> int:
@@ -61,8 +65,8 @@ class LatentCachePool:
 
     @staticmethod
     def bytes_per_block(spec: HybridSpec, block_size: int, dtype) -> int:
-        w = sum(ls.mixer.cache_width for ls in spec.layers
-                if LatentCachePool._owns_rows(ls.mixer))
+        w = sum(m.cache_width for _, m in mixer_units(spec)
+                if LatentCachePool._owns_rows(m))
         return max(1, w) * block_size * torch.tensor([], dtype=dtype).element_size()
 
     def copy_block(self, src: int, dst: int) -> None:
@@ -80,19 +84,19 @@ class StateSlotPool:
         self.tails: List[torch.Tensor] = [
             torch.zeros(num_slots + 1, k, D, dtype=torch.float32, device=device)
             for _ in spec.layers]
-        # recurrent state: layer index -> [slots + 1, state size] fp32
-        self.recurrent: Dict[int, torch.Tensor] = {
-            i: torch.zeros(num_slots + 1, ls.mixer.state_size, dtype=torch.float32,
+        # recurrent state: mixer unit -> [slots + 1, state size] fp32
+        self.recurrent: Dict[object, torch.Tensor] = {
+            i: torch.zeros(num_slots + 1, m.state_size, dtype=torch.float32,
                            device=device)
-            for i, ls in enumerate(spec.layers)
-            if isinstance(ls.mixer, (MinGRUSpec, DeltaRuleSpec))}
-        # a mixer's own short convolution: layer index ->
+            for i, m in mixer_units(spec)
+            if isinstance(m, (MinGRUSpec, DeltaRuleSpec))}
+        # a mixer's own short convolution: mixer unit ->
         # [slots + 1, taps - 1, channels] fp32
-        self.mixer_tails: Dict[int, torch.Tensor] = {
-            i: torch.zeros(num_slots + 1, ls.mixer.taps - 1, ls.mixer.conv_channels,
+        self.mixer_tails: Dict[object, torch.Tensor] = {
+            i: torch.zeros(num_slots + 1, m.taps - 1, m.conv_channels,
                            dtype=torch.float32, device=device)
-            for i, ls in enumerate(spec.layers)
-            if isinstance(ls.mixer, DeltaRuleSpec)}
+            for i, m in mixer_units(spec)
+            if isinstance(m, DeltaRuleSpec)}
         self._free = list(range(num_slots - 1, -1, -1))
 
     @property

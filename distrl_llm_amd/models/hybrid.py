@@ -38,6 +38,22 @@ parameter, so another design can reuse them in another order.
   router takes a softmax over all outputs, chooses with an added
   correction, scales the unnormalised scores, may name identity experts
   and adds an always-on shared expert.
+
+``Kakilorn`` is the third:
+
+* residual stream in fp32, sublayers read it as it is and only their
+  output is normed (post-norm arrangement, plain norm weights):
+  ``x += norm(mixer(x))`` then ``x += norm(ff(x))``; the embedding is
+  scaled and also serves, scaled again, as the output matrix;
+* mixers: latent attention with low-rank queries, interleaved-pair rotary
+  whose frequencies are rescaled for long contexts, a per-head sink in the
+  softmax and a per-head sigmoid output gate; the gated delta rule with a
+  decay per head *and key channel* (low-rank decay input, low-rank sigmoid
+  output gate); and a parallel pair read from the same input: sigmoid
+  attention (no softmax; RMS-normed q/k, a linear distance penalty per
+  head, a sliding window that also keeps the first tokens) beside the
+  per-head gated delta rule, summed with fixed scales;
+* feed-forward: a dense SiLU-gated GLU.
 """
 
 from __future__ import annotations
@@ -66,8 +82,27 @@ class LatentAttentionSpec:
     rope_dims: int      # how many of the rot_dim entries are rotated
     window: int         # 0 = unbounded causal
     kv_from: Optional[int] = None   # layer whose cache this layer reads
+    q_rank: int = 0     # > 0: queries go through a normed latent of this size
+    rope_pairs: bool = False        # rotate entries (2i, 2i+1), else (i, i + dims/2)
+    # long-context frequency rescaling: (factor, original length, fast turns,
+    # slow turns), None = plain frequencies
+    rope_scaling: Optional[tuple] = None
+    sink: bool = False  # a learned per-head term in the softmax denominator
+    out_gate: bool = False          # per-head sigmoid gate read from the mixer input
 
     kind = "latent_attention"
+
+    @property
+    def in_size(self) -> int:
+        """Rows of the packed projection of the mixer input."""
+        n = self.q_rank if self.q_rank else self.q_size
+        if self.kv_from is None:
+            n += self.cache_width
+        return n + (self.heads if self.out_gate else 0)
+
+    def rope_table(self):
+        """(per-pair frequencies, factor on cos and sin) in double precision."""
+        return rotary_frequencies(self.rope_dims, self.rope_base, self.rope_scaling)
 
     @property
     def q_size(self) -> int:
@@ -105,6 +140,10 @@ class SinkAttentionSpec:
     kind = "sink_attention"
 
     @property
+    def in_size(self) -> int:
+        return self.q_size + self.cache_width
+
+    @property
     def q_size(self) -> int:
         return self.heads * self.dim
 
@@ -129,8 +168,23 @@ class DeltaRuleSpec:
     dim: int
     vdim: int
     taps: int
+    # decay "head": one per head from a [H, D] projection; "channel": one per
+    # head and key channel through a low-rank pair of projections
+    decay: str = "head"
+    decay_rank: int = 0
+    # output gate: "silu" of a full projection, or "sigmoid" of a low-rank pair
+    gate: str = "silu"
+    gate_rank: int = 0
 
     kind = "delta_rule"
+
+    @property
+    def in_size(self) -> int:
+        return self.conv_channels + (self.gate_rank if self.gate_rank else self.v_size)
+
+    @property
+    def ab_rows(self) -> int:           # fp32 rows: write strength | decay input
+        return self.heads + (self.decay_rank if self.decay == "channel" else self.heads)
 
     @property
     def qk_size(self) -> int:
@@ -150,11 +204,107 @@ class DeltaRuleSpec:
 
 
 @dataclass(frozen=True)
+class SigmoidAttentionSpec:
+    """Grouped-query attention whose weights are sigmoids of the scores (no
+    normalisation over keys), with RMS-normed queries and keys, a linear
+    distance penalty ``2^(-slope_exp (h+1) / H) * (i - j)`` per head, and a
+    sliding window that also keeps the first ``keep_first`` tokens."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int         # 0 = unbounded causal
+    keep_first: int
+    slope_exp: float = 8.0
+
+    kind = "sigmoid_attention"
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def k_size(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def v_size(self) -> int:
+        return self.kv_heads * self.vdim
+
+    @property
+    def in_size(self) -> int:
+        return self.q_size + self.k_size + self.v_size
+
+    @property
+    def cache_width(self) -> int:      # one cache row = [k heads | v heads]
+        return self.k_size + self.v_size
+
+    def slopes(self):
+        return [2.0 ** (-self.slope_exp * (h + 1) / self.heads)
+                for h in range(self.heads)]
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers that read the same input; the result is
+    ``left_scale * left + right_scale * right``."""
+    left: object
+    right: object
+    left_scale: float
+    right_scale: float
+
+    kind = "parallel"
+
+    @property
+    def in_size(self) -> int:
+        return self.left.in_size + self.right.in_size
+
+
+def mixer_units(spec: "HybridSpec"):
+    """Every mixer that owns cache rows or state, with its key: the layer
+    index, or (layer index, side) for the sides of a parallel pair."""
+    for i, ls in enumerate(spec.layers):
+        m = ls.mixer
+        if isinstance(m, ParallelMixerSpec):
+            yield (i, 0), m.left
+            yield (i, 1), m.right
+        else:
+            yield i, m
+
+
+def rotary_frequencies(dims: int, base: float, scaling: Optional[tuple] = None):
+    """Per-pair rotary frequencies ``base^(-2i/dims)`` and the factor on cos
+    and sin. With ``scaling = (factor, original, fast, slow)`` the pairs
+    that turn fewer than ``slow`` times over ``original`` positions are
+    slowed by ``factor``, those that turn more than ``fast`` times are kept,
+    the ones between are blended linearly over the pair index, and cos/sin
+    grow by ``0.1 ln(factor) + 1``."""
+    half = dims // 2
+    f = [float(base) ** (-2.0 * i / dims) for i in range(half)]
+    if not scaling:
+        return f, 1.0
+    factor, original, fast, slow = (float(v) for v in scaling)
+
+    def pair_of(turns):
+        return dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(base))
+
+    lo = max(math.floor(pair_of(fast)), 0)
+    hi = min(math.ceil(pair_of(slow)), dims - 1)
+    for i in range(half):
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        f[i] = f[i] / factor * ramp + f[i] * (1.0 - ramp)
+    return f, 0.1 * math.log(factor) + 1.0
+
+
+@dataclass(frozen=True)
 class GluSpec:
-    """Clamped GLU: g = min(gate, limit), u = clamp(up, +-limit),
-    y = g * sigmoid(1.702 g) * (u + 1)."""
+    """Gated linear unit. ``act`` "capped": g = min(gate, limit),
+    u = clamp(up, +-limit), y = g * sigmoid(1.702 g) * (u + 1); "silu":
+    y = silu(gate) * up (limit unused)."""
     ff: int
-    limit: float
+    limit: float = 0.0
+    act: str = "capped"
 
 
 @dataclass(frozen=True)
@@ -187,9 +337,14 @@ class HybridSpec:
     conv_taps: int
     layers: tuple = field(default_factory=tuple)
     # "parallel_gated": one norm feeds mixer and feed-forward, gated sum;
-    # "sandwich": norm before and after each sublayer, one after the other
+    # "sandwich": norm before and after each sublayer, one after the other;
+    # "post_norm": sublayers read the residual, only their output is normed
     block: str = "parallel_gated"
     design: str = "nibalix"
+    norm_offset: float = 1.0    # norm weights act as (offset + w)
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+    tied_head: bool = False     # the embedding table is the output matrix
 
     @property
     def num_layers(self) -> int:
@@ -284,6 +439,51 @@ def nibalix_config_from_spec(spec: HybridSpec) -> dict:
 
 # ---------------------------------------------------------------- weights
 
+def _make_mixer_weights(mod, m, D, P, packed_input=True):
+    """Create one mixer's packed parameters as attributes of ``mod``.
+    ``packed_input`` False: the projection of the mixer input is owned by
+    the caller (the sides of a parallel pair share one)."""
+    f32 = torch.float32
+    if packed_input:
+        mod.in_w = P(m.in_size if hasattr(m, "in_size") else 3 * m.width, D)
+    if isinstance(m, LatentAttentionSpec):
+        if m.kv_from is None:
+            mod.latent_norm_w = P(m.kv_rank, dt=f32)
+        if m.q_rank:
+            mod.q_norm_w = P(m.q_rank, dt=f32)
+            mod.uq = P(m.q_size, m.q_rank)
+        if m.sink:
+            mod.sink = P(m.heads, dt=f32)
+        mod.uk = P(m.heads, m.dim, m.kv_rank)
+        mod.uv = P(m.heads, m.vdim, m.kv_rank)
+        mod.out_w = P(D, m.heads * m.vdim)
+    elif isinstance(m, SinkAttentionSpec):
+        mod.talk = P(m.heads, m.heads, dt=f32)
+        mod.sink = P(m.heads, dt=f32)
+        mod.vmix = P(1, dt=f32)
+        mod.out_w = P(D, m.heads * m.vdim)
+    elif isinstance(m, SigmoidAttentionSpec):
+        mod.q_norm_w, mod.k_norm_w = P(m.dim, dt=f32), P(m.dim, dt=f32)
+        mod.pos_bias = P(m.heads, dt=f32)
+        mod.out_w = P(D, m.heads * m.vdim)
+    elif isinstance(m, DeltaRuleSpec):
+        mod.conv_w = P(m.conv_channels, m.taps, dt=f32)
+        mod.ab_w = P(m.ab_rows, D, dt=f32)      # [write strength; decay input]
+        mod.a_log = P(m.heads, dt=f32)
+        if m.decay == "channel":
+            mod.decay_up = P(m.heads * m.dim, m.decay_rank, dt=f32)
+            mod.dt_bias = P(m.heads * m.dim, dt=f32)
+        else:
+            mod.dt_bias = P(m.heads, dt=f32)
+        if m.gate_rank:
+            mod.gate_up = P(m.v_size, m.gate_rank)
+        mod.onorm_w = P(m.vdim, dt=f32)
+        mod.out_w = P(D, m.v_size)
+    else:
+        mod.in_b = P(3 * m.width, dt=f32)
+        mod.out_w = P(D, m.width)
+
+
 class HybridLayer(nn.Module):
     """Packed inference weights of one layer.
 
@@ -303,41 +503,30 @@ class HybridLayer(nn.Module):
                                 requires_grad=False)
 
         f32 = torch.float32
-        self.norm_w = P(D, dt=f32)
-        if spec.block == "sandwich":
+        if spec.block == "post_norm":
+            self.post_w = P(D, dt=f32)
+            if ls.mlp is not None:
+                self.ff_post_w = P(D, dt=f32)
+        elif spec.block == "sandwich":
+            self.norm_w = P(D, dt=f32)
             self.post_w = P(D, dt=f32)
             if ls.mlp is not None:
                 self.ff_norm_w, self.ff_post_w = P(D, dt=f32), P(D, dt=f32)
         else:
+            self.norm_w = P(D, dt=f32)
             if spec.conv_taps:  # 0: the mixer reads the normed input as it is
                 self.conv_w = P(D, spec.conv_taps, dt=f32)
             n_gate = 2 * D if ls.mlp is not None else D
             self.gate_w, self.gate_b = P(n_gate, D), P(n_gate, dt=f32)
         m = ls.mixer
-        if isinstance(m, LatentAttentionSpec):
-            own = m.kv_from is None
-            self.in_w = P(m.q_size + (m.cache_width if own else 0), D)
-            if own:
-                self.latent_norm_w = P(m.kv_rank, dt=f32)
-            self.uk = P(m.heads, m.dim, m.kv_rank)
-            self.uv = P(m.heads, m.vdim, m.kv_rank)
-            self.out_w = P(D, m.heads * m.vdim)
-        elif isinstance(m, SinkAttentionSpec):
-            self.in_w = P(m.q_size + m.cache_width, D)
-            self.talk = P(m.heads, m.heads, dt=f32)
-            self.sink = P(m.heads, dt=f32)
-            self.vmix = P(1, dt=f32)
-            self.out_w = P(D, m.heads * m.vdim)
-        elif isinstance(m, DeltaRuleSpec):
-            self.in_w = P(m.conv_channels + m.v_size, D)
-            self.conv_w = P(m.conv_channels, m.taps, dt=f32)
-            self.ab_w = P(2 * m.heads, D, dt=f32)       # [write strength; step]
-            self.a_log, self.dt_bias = P(m.heads, dt=f32), P(m.heads, dt=f32)
-            self.onorm_w = P(m.vdim, dt=f32)
-            self.out_w = P(D, m.v_size)
+        if isinstance(m, ParallelMixerSpec):
+            # both sides read one packed projection of the shared input
+            self.in_w = P(m.in_size, D)
+            self.left, self.right = nn.Module(), nn.Module()
+            _make_mixer_weights(self.left, m.left, D, P, packed_input=False)
+            _make_mixer_weights(self.right, m.right, D, P, packed_input=False)
         else:
-            self.in_w, self.in_b = P(3 * m.width, D), P(3 * m.width, dt=f32)
-            self.out_w = P(D, m.width)
+            _make_mixer_weights(self, m, D, P)
         f = ls.mlp
         if isinstance(f, GluSpec):
             self.gu_w, self.down_w = P(2 * f.ff, D), P(D, f.ff)
@@ -373,7 +562,8 @@ class HybridLM(nn.Module):
         if spec.design == "nibalix":
             self.embed_norm_w = P(D, dt=f32)
         self.final_norm_w = P(D, dt=f32)
-        self.head = P(spec.vocab_size, D)
+        # a tied output matrix is the embedding parameter itself
+        self.head = self.embed if spec.tied_head else P(spec.vocab_size, D)
         self.layers = nn.ModuleList(
             [HybridLayer(spec, ls, dtype, device) for ls in spec.layers])
 
@@ -389,6 +579,8 @@ class HybridLM(nn.Module):
         entries carry an index tuple instead of a row range."""
         if self.spec.design == "nedasun":
             return _nedasun_named_slices(self)
+        if self.spec.design == "kakilorn":
+            return _kakilorn_named_slices(self)
         out = {"embed": (self.embed, None), "embed.norm": (self.embed_norm_w, None),
                "final.norm": (self.final_norm_w, None), "head": (self.head, None)}
         D = self.spec.width
@@ -480,7 +672,9 @@ class HybridLM(nn.Module):
                 r *= 0.5
             elif dst.dim() >= 2 and "canon" not in name:
                 r *= 1.0 / math.sqrt(dst.shape[-1])
-            elif name.endswith("dkv.norm") or name.endswith("mix.norm"):
+            elif (name.endswith("dkv.norm") or name.endswith("mix.norm")
+                  or (self.spec.norm_offset == 0.0 and last in
+                      ("norm", "norm1", "norm2"))):
                 r = 1.0 + 0.1 * r
             else:
                 r *= 0.1
@@ -690,3 +884,218 @@ def save_nedasun_checkpoint(model: HybridLM, path: str) -> None:
     save_file(model.export_tensors(), os.path.join(path, "model.safetensors"))
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(nedasun_config_from_spec(model.spec), f, indent=1)
+
+
+# --------------------------------------------------------------- Kakilorn
+
+def _delta_from_config(i, mc, channel: bool) -> DeltaRuleSpec:
+    heads, kvh = int(mc["heads"]), int(mc["kv_heads"])
+    if kvh < 1 or heads % kvh:
+        raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+    if int(mc["conv"]) < 1:
+        raise ValueError(f"layer {i}: conv needs at least one tap")
+    return DeltaRuleSpec(heads=heads, kv_heads=kvh, dim=int(mc["dim"]),
+                         vdim=int(mc["vdim"]), taps=int(mc["conv"]),
+                         decay="channel" if channel else "head",
+                         gate="sigmoid" if channel else "silu")
+
+
+def kakilorn_spec_from_config(cfg: dict, name: str = "kakilorn",
+                              shapes: Optional[dict] = None) -> HybridSpec:
+    """Map a Kakilorn ``config.json`` onto the generic layer specs. The
+    ranks of the low-rank decay and gate inputs are not in the config: they
+    are the row counts of the checkpoint's ``a1``/``g1`` tensors
+    (``shapes``: tensor name -> shape), or ``decay_rank``/``gate_rank``
+    entries of the mixer's config when a checkpoint is written from a spec."""
+    shapes = shapes or {}
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc, typ = lc["mixer"], lc["type"]
+        if typ == "latent_attention":
+            rot = mc.get("rot") or {}
+            sc = rot.get("scaling")
+            mixer = LatentAttentionSpec(
+                heads=int(mc["heads"]), dim=int(mc["dim"]),
+                rot_dim=int(mc["rot_dim"]), vdim=int(mc["vdim"]),
+                kv_rank=int(mc["kv_rank"]), scale=float(mc["scale"]),
+                rope_base=float(rot.get("base") or 10000.0),
+                rope_dims=int(rot["dims"] if rot.get("dims") is not None
+                              else mc["rot_dim"]),
+                window=0, q_rank=int(mc["q_rank"]), rope_pairs=True,
+                rope_scaling=(None if not sc else
+                              (float(sc["factor"]), float(sc["original"]),
+                               float(sc["fast"]), float(sc["slow"]))),
+                sink=True, out_gate=True)
+            if mixer.rope_dims > mixer.rot_dim or mixer.rope_dims % 2:
+                raise ValueError(f"layer {i}: rot.dims must be even and <= rot_dim")
+            if mixer.q_rank < 1:
+                raise ValueError(f"layer {i}: q_rank must be positive")
+        elif typ == "channel_delta":
+            d = _delta_from_config(i, mc, True)
+            ra = shapes.get(f"l{i}.mix.a1", (mc.get("decay_rank"),))[0]
+            rg = shapes.get(f"l{i}.mix.g1", (mc.get("gate_rank"),))[0]
+            if not ra or not rg:
+                raise ValueError(f"layer {i}: the ranks of the decay and gate "
+                                 f"inputs are unknown")
+            mixer = DeltaRuleSpec(**{**d.__dict__, "decay_rank": int(ra),
+                                     "gate_rank": int(rg)})
+        elif typ == "parallel":
+            lm, rm = mc["left"], mc["right"]
+            heads, kvh = int(lm["heads"]), int(lm["kv_heads"])
+            if kvh < 1 or heads % kvh:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            mask = lm.get("mask") or {}
+            left = SigmoidAttentionSpec(
+                heads=heads, kv_heads=kvh, dim=int(lm["dim"]),
+                vdim=int(lm["vdim"]), scale=float(lm["scale"]),
+                window=int(mask.get("size") or 0),
+                keep_first=int(mask.get("keep_first") or 0))
+            mixer = ParallelMixerSpec(left, _delta_from_config(i, rm, False),
+                                      float(mc["left_scale"]),
+                                      float(mc["right_scale"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {typ!r}")
+        fc, mlp = lc.get("mlp"), None
+        if fc is not None:
+            if fc.get("kind") != "dense":
+                raise ValueError(f"layer {i}: unknown mlp kind {fc.get('kind')!r}")
+            mlp = GluSpec(ff=int(fc["ff"]), act="silu")
+        layers.append(LayerSpec(mixer, mlp))
+    return HybridSpec(name=name, vocab_size=int(cfg["vocab"]),
+                      width=int(cfg["width"]),
+                      norm_eps=float(cfg["norm"]["eps"]), residual_mult=1.0,
+                      conv_taps=0, layers=tuple(layers), block="post_norm",
+                      design="kakilorn", norm_offset=0.0,
+                      embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+                      logit_scale=float(cfg.get("logit_scale", 1.0)),
+                      tied_head=True)
+
+
+def kakilorn_config_from_spec(spec: HybridSpec) -> dict:
+    """Inverse of :func:`kakilorn_spec_from_config` (checkpoint saving)."""
+    def delta(m):
+        return {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+                "vdim": m.vdim, "conv": m.taps}
+
+    layers = []
+    for ls in spec.layers:
+        m = ls.mixer
+        if isinstance(m, LatentAttentionSpec):
+            rot = {"base": m.rope_base, "dims": m.rope_dims}
+            if m.rope_scaling:
+                rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"),
+                                          m.rope_scaling))
+            mc = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim,
+                  "vdim": m.vdim, "kv_rank": m.kv_rank, "q_rank": m.q_rank,
+                  "scale": m.scale, "rot": rot}
+            typ = "latent_attention"
+        elif isinstance(m, DeltaRuleSpec):
+            mc, typ = delta(m), "channel_delta"
+        else:
+            a = m.left
+            left = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim,
+                    "vdim": a.vdim, "scale": a.scale}
+            if a.window:
+                left["mask"] = {"size": a.window, "keep_first": a.keep_first}
+            mc = {"left": left, "right": delta(m.right),
+                  "left_scale": m.left_scale, "right_scale": m.right_scale}
+            typ = "parallel"
+        fc = None if ls.mlp is None else {"kind": "dense", "ff": ls.mlp.ff}
+        layers.append({"type": typ, "mixer": mc, "mlp": fc})
+    return {"architecture": "Kakilorn", "embedding": {"scale": spec.embed_scale},
+            "layers": layers, "logit_scale": spec.logit_scale,
+            "norm": {"eps": spec.norm_eps}, "vocab": spec.vocab_size,
+            "width": spec.width}
+
+
+def _kakilorn_named_slices(model: "HybridLM") -> Dict[str, tuple]:
+    out = {"embed": (model.embed, None), "final.norm": (model.final_norm_w, None)}
+
+    def delta(x, m, W, in_w, r0):
+        """Names of a delta-rule mixer whose packed input rows start at r0."""
+        n, nv = m.qk_size, m.v_size
+        for nm, a, rows in (("q", 0, n), ("k", n, n), ("v", 2 * n, nv)):
+            out[x + nm] = (in_w, (r0 + a, rows))
+            out[x + nm + ".conv"] = (W.conv_w, (a, rows))
+        c = r0 + m.conv_channels
+        out[x + "b"] = (W.ab_w, (0, m.heads))
+        if m.decay == "channel":
+            out[x + "a1"] = (W.ab_w, (m.heads, m.decay_rank))
+            out[x + "a2"] = (W.decay_up, None)
+        else:
+            out[x + "a"] = (W.ab_w, (m.heads, m.heads))
+        if m.gate_rank:
+            out[x + "g1"] = (in_w, (c, m.gate_rank))
+            out[x + "g2"] = (W.gate_up, None)
+        else:
+            out[x + "g"] = (in_w, (c, nv))
+        out[x + "A_log"], out[x + "dt_bias"] = (W.a_log, None), (W.dt_bias, None)
+        out[x + "norm"], out[x + "o"] = (W.onorm_w, None), (W.out_w, None)
+
+    for i, (ls, L) in enumerate(zip(model.spec.layers, model.layers)):
+        p, m = f"l{i}.", ls.mixer
+        x = p + "mix."
+        out[p + "norm1"] = (L.post_w, None)
+        if isinstance(m, LatentAttentionSpec):
+            w = m.cache_width
+            out[x + "dq"] = (L.in_w, (0, m.q_rank))
+            out[x + "dkv"] = (L.in_w, (m.q_rank, w))
+            out[x + "g"] = (L.in_w, (m.q_rank + w, m.heads))
+            out[x + "dq.norm"], out[x + "uq"] = (L.q_norm_w, None), (L.uq, None)
+            out[x + "dkv.norm"] = (L.latent_norm_w, None)
+            out[x + "uk"], out[x + "uv"] = (L.uk, "flat"), (L.uv, "flat")
+            out[x + "sink"], out[x + "o"] = (L.sink, None), (L.out_w, None)
+        elif isinstance(m, DeltaRuleSpec):
+            delta(x, m, L, L.in_w, 0)
+        else:
+            a, W = m.left, L.left
+            y = x + "left."
+            out[y + "q"] = (L.in_w, (0, a.q_size))
+            out[y + "k"] = (L.in_w, (a.q_size, a.k_size))
+            out[y + "v"] = (L.in_w, (a.q_size + a.k_size, a.v_size))
+            out[y + "q.norm"], out[y + "k.norm"] = (W.q_norm_w, None), (W.k_norm_w, None)
+            out[y + "pb"], out[y + "o"] = (W.pos_bias, None), (W.out_w, None)
+            delta(x + "right.", m.right, L.right, L.in_w, a.in_size)
+        if ls.mlp is not None:
+            f = ls.mlp
+            out[p + "norm2"] = (L.ff_post_w, None)
+            out[p + "mlp.gate"] = (L.gu_w, (0, f.ff))
+            out[p + "mlp.up"] = (L.gu_w, (f.ff, f.ff))
+            out[p + "mlp.down"] = (L.down_w, None)
+    return out
+
+
+def _safetensors_shapes(path: str) -> dict:
+    """Tensor name -> shape from a safetensors file's header."""
+    import struct
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        head = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in head.items() if k != "__metadata__"}
+
+
+def load_kakilorn_checkpoint(path: str, dtype=torch.bfloat16, device=None) -> HybridLM:
+    from safetensors.torch import load_file
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    name = os.path.basename(os.path.normpath(path)) or "kakilorn"
+    file = os.path.join(path, "model.safetensors")
+    spec = kakilorn_spec_from_config(cfg, name, _safetensors_shapes(file))
+    model = HybridLM(spec, dtype=dtype, device=device)
+    tensors = load_file(file)
+    known = model._named_slices()
+    extra = sorted(k for k in tensors if k not in known)
+    if extra:
+        import sys
+        sys.stderr.write(f"[kakilorn] ignoring {len(extra)} tensors the design "
+                         f"does not name: {extra[:4]}\n")
+    model.load_tensors({k: v for k, v in tensors.items() if k in known})
+    return model
+
+
+def save_kakilorn_checkpoint(model: HybridLM, path: str) -> None:
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    save_file(model.export_tensors(), os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(kakilorn_config_from_spec(model.spec), f, indent=1)

@@ -69,9 +69,11 @@ def load_model_and_engine(path_or_name: str, engine_cfg, dtype=None,
 
 
 def _register_builtin():
-    from .hybrid import load_nedasun_checkpoint, load_nibalix_checkpoint
+    from .hybrid import (load_kakilorn_checkpoint, load_nedasun_checkpoint,
+                         load_nibalix_checkpoint)
     register_hybrid_design("Nibalix", load_nibalix_checkpoint)
     register_hybrid_design("Nedasun", load_nedasun_checkpoint)
+    register_hybrid_design("Kakilorn", load_kakilorn_checkpoint)
 
 
 _register_builtin()

@@ -31,11 +31,12 @@ def _bf16(dtype) -> bool:
     return dtype == torch.bfloat16
 
 
-def offset_rmsnorm(x, w, eps, out_dtype):
+def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0):
+    """x / rms(x) * (offset + w) -> (fp32, out_dtype) rows."""
     if x.is_cuda:
         return _ext("offset_rmsnorm").offset_rmsnorm(x.contiguous(), w, eps,
-                                                     _bf16(out_dtype))
-    return R.offset_rmsnorm(x, w, eps, out_dtype)
+                                                     _bf16(out_dtype), offset)
+    return R.offset_rmsnorm(x, w, eps, out_dtype, offset)
 
 
 def causal_tap_conv(h, w, tails, cu, tok_seq, slots, out_dtype):
@@ -45,15 +46,20 @@ def causal_tap_conv(h, w, tails, cu, tok_seq, slots, out_dtype):
     return R.causal_tap_conv(h, w, tails, cu, slots, out_dtype)
 
 
-def latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
-                   positions, rope_base, rope_dims, page_slot, cache):
-    if proj.is_cuda:
+def latent_prepare(q, dkv, heads, dim, rot_dim, kv_rank, norm_w, eps,
+                   positions, rope_base, rope_dims, page_slot, cache,
+                   freqs=None, mag=1.0, pairs=False):
+    """``q`` and ``dkv`` may be column slices of wider row-major matrices;
+    ``dkv`` None: the layer reads another layer's cache. ``freqs`` (fp32
+    [rope_dims / 2]) with ``mag`` and ``pairs`` selects a tabulated rotation
+    (rescaled frequencies, cos/sin factor, (2i, 2i+1) pairs)."""
+    if q.is_cuda:
         return _ext("latent_prepare").latent_prepare(
-            proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
-            positions, rope_base, rope_dims, page_slot, cache)
-    return R.latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache,
-                            norm_w, eps, positions, rope_base, rope_dims,
-                            page_slot, cache)
+            q, dkv, heads, dim, rot_dim, kv_rank, norm_w, eps, positions,
+            rope_base, rope_dims, page_slot, cache, freqs, mag, pairs)
+    return R.latent_prepare(q, dkv, heads, dim, rot_dim, kv_rank, norm_w, eps,
+                            positions, rope_base, rope_dims, page_slot, cache,
+                            freqs, mag, pairs)
 
 
 QUERY_TILE = 16   # most queries of one sequence the tiled kernel takes at once
@@ -74,17 +80,21 @@ def query_tiles(row_lengths, tile=QUERY_TILE):
 
 def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                             block_size, cu, tok_seq, positions, window, scale,
-                            out_dtype, tiles=None, max_tile=0):
+                            out_dtype, tiles=None, max_tile=0, sink=None,
+                            gate=None):
     """``tiles`` (int32 [n, 3] from :func:`query_tiles`, with ``max_tile``)
     selects the tiled MFMA kernel for bf16; without it, or in fp32, the
-    one-wave-per-query kernel runs."""
+    one-wave-per-query kernel runs. ``sink`` (fp32 [H]) joins the softmax
+    denominator; ``gate`` ([T, H] pre-activations, may be a column slice)
+    scales head h's result by its sigmoid."""
     if q_lat.is_cuda:
         return _ext("latent_window_attention").latent_window_attention(
             q_lat.contiguous(), q_rot, cache, kv_rank, block_tables,
-            block_size, tok_seq, positions, window, scale, tiles, max_tile)
+            block_size, tok_seq, positions, window, scale, tiles, max_tile,
+            sink, gate)
     return R.latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                                      block_size, cu, positions, window, scale,
-                                     out_dtype)
+                                     out_dtype, sink, gate)
 
 
 SCAN_CHUNK = 64    # tokens per parallel chunk of a long row's recurrence
@@ -152,15 +162,24 @@ def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
 
 # ------------------------------------------------- sandwich-block mechanisms
 
-def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
-    """Fused sublayer tail: x += rms_unit(y [+ y2]) * (1 + post_w) on the
-    fp32 residual (in place), then, with ``next_w``, the next offset RMS
-    norm of the new residual in ``out_dtype``; None without."""
+def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
+                           offset=1.0, y_scale=1.0, y2_scale=1.0,
+                           cast_next=False):
+    """Fused sublayer tail: x += rms_unit(y_scale y [+ y2_scale y2]) *
+    (offset + post_w) on the fp32 residual (in place), then, with
+    ``next_w``, the next offset RMS norm of the new residual in
+    ``out_dtype``; with ``cast_next`` instead the new residual itself in
+    ``out_dtype`` (x when that is fp32); None without either."""
     if x.is_cuda:
-        return _ext("sandwich_residual_norm").sandwich_residual_norm(
+        h = _ext("sandwich_residual_norm").sandwich_residual_norm(
             x, y.contiguous(), None if y2 is None else y2.contiguous(), post_w,
-            next_w, eps, _bf16(out_dtype))
-    return R.sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype)
+            next_w, eps, _bf16(out_dtype), offset, y_scale, y2_scale,
+            cast_next and next_w is None and _bf16(out_dtype))
+        if h is None and cast_next and next_w is None:
+            return x
+        return h
+    return R.sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
+                                    offset, y_scale, y2_scale, cast_next)
 
 
 def rope_kv_write(proj, heads, kv_heads, dim, vdim, positions, rope_base,
@@ -200,24 +219,62 @@ def tap_conv_silu(x, w, tails, cu, tok_seq, slots, out_dtype):
 
 def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
                      slots, heads, kv_heads, dim, vdim, out_dtype, h=None,
-                     ab_w=None):
-    """``ab`` None: the [strength | step] inputs are projected inside the op
-    from the mixer input ``h`` with the fp32 matrix ``ab_w`` [2H, D]."""
+                     ab_w=None, decay_up=None, gate_sigmoid=False):
+    """``ab`` None: the [strength | decay input] rows are projected inside
+    the op from the mixer input ``h`` with the fp32 matrix ``ab_w``.
+    ``decay_up`` (fp32 [H dim, R]): a decay per head and key channel from the
+    R low-rank decay inputs, ``dt_bias`` [H dim]; else one decay per head.
+    ``gate_sigmoid``: sigmoid output gate instead of SiLU."""
     if qkv.is_cuda:
         return _ext("gated_delta_rule").gated_delta_rule(
             qkv, gate, ab, h, ab_w, a_log, dt_bias, onorm_w, eps, state, cu,
-            slots, heads, kv_heads, dim, vdim)
+            slots, heads, kv_heads, dim, vdim, decay_up, gate_sigmoid)
     if ab is None:
         ab = torch.nn.functional.linear(h.float(), ab_w.float())
     return R.gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps,
                               state, cu, slots, heads, kv_heads, dim, vdim,
-                              out_dtype)
+                              out_dtype, decay_up, gate_sigmoid)
 
 
 def capped_glu(gu, limit):
     if gu.is_cuda:
         return _ext("capped_glu").capped_glu(gu, limit)
     return R.capped_glu(gu, limit)
+
+
+def silu_glu(gu):
+    """Rows [gate | up] -> silu(gate) * up."""
+    if gu.is_cuda:
+        return _ext("silu_glu").silu_glu(gu)
+    return R.silu_glu(gu)
+
+
+def qk_norm_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w, eps,
+                     page_slot, cache):
+    """``proj`` rows [q | k | v] may be a column slice of a wider matrix."""
+    if proj.is_cuda:
+        return _ext("qk_norm_kv_write").qk_norm_kv_write(
+            proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w, eps,
+            page_slot, cache)
+    return R.qk_norm_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w,
+                              k_norm_w, eps, page_slot, cache)
+
+
+def sigmoid_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
+                      block_size, cu, tok_seq, positions, scale, window,
+                      keep_first, slopes, pos_bias, out_dtype, tiles=None,
+                      max_tile=0):
+    """``tiles`` (from :func:`query_tiles` with ``WIDE_QUERY_TILE``) selects
+    the tiled MFMA kernel for bf16 prompt portions; other steps and fp32
+    models run one wave per (token, head)."""
+    if q.is_cuda:
+        return _ext("sigmoid_attention").sigmoid_attention(
+            q, cache, heads, kv_heads, dim, vdim, block_tables, block_size,
+            tok_seq, positions, scale, window, keep_first, slopes, pos_bias,
+            tiles, max_tile)
+    return R.sigmoid_attention(q, cache, heads, kv_heads, dim, vdim,
+                               block_tables, block_size, cu, positions, scale,
+                               window, keep_first, slopes, pos_bias, out_dtype)
 
 
 def moe_route_all(h, router_w, correction, top, scale):

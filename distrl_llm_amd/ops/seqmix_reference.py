@@ -18,10 +18,10 @@ import torch
 import torch.nn.functional as F
 
 
-def offset_rmsnorm(x, w, eps, out_dtype):
-    """x / sqrt(mean(x^2) + eps) * (1 + w) in fp32 -> (fp32, out_dtype)."""
+def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0):
+    """x / sqrt(mean(x^2) + eps) * (offset + w) in fp32 -> (fp32, out_dtype)."""
     x = x.float()
-    h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float())
+    h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
     return h, h.to(out_dtype)
 
 
@@ -62,35 +62,65 @@ def _rotate_half(v, positions, base, dims):
     return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], -1)
 
 
-def latent_prepare(proj, heads, dim, rot_dim, kv_rank, own_cache, norm_w, eps,
-                   positions, rope_base, rope_dims, page_slot, cache):
-    """From the packed [q | dkv] projection rows: write the normed latent
-    and the rotated shared key part into ``cache`` rows ``page_slot``
-    (layers with a cache of their own), and return the rotated query part
-    [T, heads, rot_dim] in fp32."""
-    T = proj.shape[0]
-    q = proj[:, :heads * (dim + rot_dim)].view(T, heads, dim + rot_dim)
-    q_rot = _rotate_half(q[..., dim:].float(), positions, rope_base, rope_dims)
-    if own_cache:
-        d = proj[:, heads * (dim + rot_dim):].float()
+def _rotate_table(v, positions, freqs, mag, pairs):
+    """Rotate the first 2 * len(freqs) entries of the last axis by the
+    angles position * freqs, cos and sin scaled by ``mag``; pairs (2i, 2i+1)
+    or (i, i + half). v fp32 [T, ..., n]."""
+    half = freqs.numel()
+    if half == 0:
+        return v
+    dims = 2 * half
+    ang = positions.to(torch.float32)[:, None] * freqs.float()[None, :]
+    shape = [v.shape[0]] + [1] * (v.dim() - 2) + [half]
+    c, s = (torch.cos(ang) * mag).view(shape), (torch.sin(ang) * mag).view(shape)
+    if pairs:
+        a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+        rot = torch.stack([a * c - b * s, b * c + a * s], -1).flatten(-2)
+        return torch.cat([rot, v[..., dims:]], -1)
+    a, b = v[..., :half], v[..., half:dims]
+    return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], -1)
+
+
+def latent_prepare(q, dkv, heads, dim, rot_dim, kv_rank, norm_w, eps,
+                   positions, rope_base, rope_dims, page_slot, cache,
+                   freqs=None, mag=1.0, pairs=False):
+    """q [T, heads * (dim + rot_dim)] query rows, dkv [T, kv_rank + rot_dim]
+    (None for a layer that reads another layer's cache): write the normed
+    latent and the rotated shared key part into ``cache`` rows
+    ``page_slot`` and return the rotated query part [T, heads, rot_dim] in
+    fp32. ``freqs`` (fp32 [rope_dims / 2]) replaces base^(-2i/dims); ``mag``
+    scales cos and sin; ``pairs`` rotates entries (2i, 2i+1) instead of
+    (i, i + dims/2)."""
+    T = q.shape[0]
+
+    def rot(v):
+        if freqs is None:
+            return _rotate_half(v, positions, rope_base, rope_dims)
+        return _rotate_table(v, positions, freqs, mag, pairs)
+
+    q = q.reshape(T, heads, dim + rot_dim)
+    q_rot = rot(q[..., dim:].float())
+    if dkv is not None:
+        d = dkv.float()
         c = d[:, :kv_rank]
         c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
-        kr = _rotate_half(d[:, kv_rank:kv_rank + rot_dim], positions,
-                          rope_base, rope_dims)
+        kr = rot(d[:, kv_rank:kv_rank + rot_dim])
         cache[page_slot.long()] = torch.cat([c, kr], -1).to(cache.dtype)
     return q_rot
 
 
 def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
                             block_size, cu, positions, window, scale,
-                            out_dtype):
+                            out_dtype, sink=None, gate=None):
     """Softmax attention in latent space over a paged cache.
 
     q_lat [H, T, kv_rank] (the query already folded through the key
     up-projection), q_rot fp32 [T, H, rot_dim], cache rows
     [c (kv_rank) | k_rot]. Token at position p sees positions j with
-    0 <= p - j < window (window 0: all j <= p). Returns sum_j p_j c_j,
-    [H, T, kv_rank]."""
+    0 <= p - j < window (window 0: all j <= p). ``sink`` (fp32 [H]) adds
+    exp(sink[h]) to the softmax denominator; ``gate`` ([T, H]
+    pre-activations) multiplies head h's result by sigmoid(gate[t, h]).
+    Returns sum_j p_j c_j, [H, T, kv_rank]."""
     H, T, r = q_lat.shape
     out = torch.zeros(H, T, r, dtype=torch.float32, device=q_lat.device)
     cu_l = cu.tolist()
@@ -113,7 +143,12 @@ def latent_window_attention(q_lat, q_rot, cache, kv_rank, block_tables,
         if window > 0:
             ok = ok & (p - j[None, :] < window)
         s = s.masked_fill(~ok[None], float("-inf"))
-        out[:, a:e] = torch.einsum("htj,jr->htr", torch.softmax(s, -1), c)
+        if sink is not None:
+            s = torch.cat([s, sink.float()[:, None, None].expand(-1, e - a, 1)], -1)
+        w = torch.softmax(s, -1)[..., :j.numel()]
+        out[:, a:e] = torch.einsum("htj,jr->htr", w, c)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float()).t()[:, :, None]
     return out.to(out_dtype)
 
 
@@ -184,16 +219,21 @@ def gated_residual_add(x, mix, ff, gates, gate_b, mult):
 
 # ------------------------------------------------- sandwich-block mechanisms
 
-def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype):
-    """x += rms_unit(y [+ y2]) * (1 + post_w) on the fp32 residual, in
-    place; with ``next_w`` also returns the next offset RMS norm of the new
-    residual in ``out_dtype``, else None."""
-    s = y.float() if y2 is None else y.float() + y2.float()
+def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
+                           offset=1.0, y_scale=1.0, y2_scale=1.0,
+                           cast_next=False):
+    """x += rms_unit(y_scale y [+ y2_scale y2]) * (offset + post_w) on the
+    fp32 residual, in place; with ``next_w`` also returns the next offset RMS
+    norm of the new residual in ``out_dtype``; with ``cast_next`` the new
+    residual itself in ``out_dtype``; else None."""
+    s = y.float() * y_scale
+    if y2 is not None:
+        s = s + y2.float() * y2_scale
     x.add_(s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps)
-           * (1.0 + post_w.float()))
-    if next_w is None:
-        return None
-    return offset_rmsnorm(x, next_w, eps, out_dtype)[1]
+           * (offset + post_w.float()))
+    if next_w is not None:
+        return offset_rmsnorm(x, next_w, eps, out_dtype, offset)[1]
+    return x.to(out_dtype) if cast_next else None
 
 
 def _rotate_pairs(v, positions, base, dims):
@@ -294,7 +334,8 @@ def tap_conv_silu(x, w, tails, cu, slots, out_dtype):
 
 
 def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
-                     slots, heads, kv_heads, dim, vdim, out_dtype):
+                     slots, heads, kv_heads, dim, vdim, out_dtype,
+                     decay_up=None, gate_sigmoid=False):
     """Gated delta rule over a flat batch.
 
     qkv [T, 2 G dim + H vdim] (after convolution and SiLU), gate [T, H vdim]
@@ -303,7 +344,12 @@ def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
     beta = sigmoid(b); decay = exp(-exp(a_log) softplus(a + dt_bias));
     S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
     out = o / rms(o) * onorm_w * silu(gate). state fp32
-    [slots, H * vdim * dim] (per head value-major: S^T), advanced in place."""
+    [slots, H * vdim * dim] (per head value-major: S^T), advanced in place.
+    With ``decay_up`` (fp32 [H dim, R]) the decay is per head and key
+    channel: ab = [write strength (H) | low-rank decay input (R)], the step
+    is softplus(decay_up a + dt_bias) with dt_bias [H dim], and the decay
+    multiplies the state's key rows. ``gate_sigmoid``: the output gate is
+    sigmoid(gate) instead of silu(gate)."""
     T = qkv.shape[0]
     H, G = heads, kv_heads
     rep = H // G
@@ -316,21 +362,28 @@ def gated_delta_rule(qkv, gate, ab, a_log, dt_bias, onorm_w, eps, state, cu,
     k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
     q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
     beta = torch.sigmoid(ab[:, :H].float())
-    decay = torch.exp(-torch.exp(a_log.float())
-                      * F.softplus(ab[:, H:].float() + dt_bias.float()))
+    if decay_up is None:
+        decay = torch.exp(-torch.exp(a_log.float())
+                          * F.softplus(ab[:, H:].float() + dt_bias.float()))
+        decay = decay[:, :, None]                       # [T, H, 1]
+    else:
+        step = F.softplus(F.linear(ab[:, H:].float(), decay_up.float())
+                          + dt_bias.float()).view(T, H, dim)
+        decay = torch.exp(-torch.exp(a_log.float())[None, :, None] * step)
     o = torch.empty(T, H, vdim, dtype=torch.float32, device=qkv.device)
     cu_l, slots_l = cu.tolist(), slots.tolist()
     for b, s in enumerate(slots_l):
         S = state[s].view(H, vdim, dim).transpose(1, 2).clone()
         for t in range(cu_l[b], cu_l[b + 1]):
-            S = decay[t][:, None, None] * S
+            S = decay[t][:, :, None] * S
             u = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
             S = S + k[t][:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hkv,hk->hv", S, q[t])
         state[s] = S.transpose(1, 2).reshape(-1)
     o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * onorm_w.float()
     g = gate.float().view(T, H, vdim)
-    return (o * g * torch.sigmoid(g)).reshape(T, H * vdim).to(out_dtype)
+    act = torch.sigmoid(g) if gate_sigmoid else g * torch.sigmoid(g)
+    return (o * act).reshape(T, H * vdim).to(out_dtype)
 
 
 def capped_glu(gu, limit):
@@ -340,6 +393,66 @@ def capped_glu(gu, limit):
     g = gu[:, :ff].float().clamp(max=limit)
     u = gu[:, ff:].float().clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(gu.dtype)
+
+
+def silu_glu(gu):
+    """gu [T, 2ff] = [gate | up]: silu(gate) * up, in gu's dtype."""
+    ff = gu.shape[1] // 2
+    g = gu[:, :ff].float()
+    return (g * torch.sigmoid(g) * gu[:, ff:].float()).to(gu.dtype)
+
+
+def qk_norm_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w, eps,
+                     page_slot, cache):
+    """From packed [q | k | v] projection rows: RMS-norm every q and k head
+    over ``dim`` with the shared plain weights, write [k | v] into ``cache``
+    rows ``page_slot``; returns the normed queries [T, heads, dim] in the
+    projection's dtype."""
+    T = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q = proj[:, :nq].float().view(T, heads, dim)
+    k = proj[:, nq:nq + nk].float().view(T, kv_heads, dim)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    v = proj[:, nq + nk:nq + nk + kv_heads * vdim].float()
+    cache[page_slot.long()] = torch.cat([k.reshape(T, nk), v], -1).to(cache.dtype)
+    return q.to(proj.dtype)
+
+
+def sigmoid_attention(q, cache, heads, kv_heads, dim, vdim, block_tables,
+                      block_size, cu, positions, scale, window, keep_first,
+                      slopes, pos_bias, out_dtype):
+    """Grouped-query attention with sigmoid weights over paged [k | v] rows.
+
+    weight(i, j) = sigmoid(q_i . k_j * scale - slopes[h] (i - j) + pos_bias[h])
+    for the visible keys j <= i with i - j < window or j < keep_first
+    (window 0: all j <= i); weights are not normalised.
+    q [T, H, dim] -> [T, H * vdim]."""
+    T = q.shape[0]
+    rep = heads // kv_heads
+    nk = kv_heads * dim
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32, device=q.device)
+    cu_l, pos_l = cu.tolist(), positions.tolist()
+    sl = slopes.float()[:, None, None]
+    for b in range(len(cu_l) - 1):
+        a, e = cu_l[b], cu_l[b + 1]
+        if e == a:
+            continue
+        j = torch.arange(0, pos_l[e - 1] + 1, device=cache.device)
+        rows = block_tables[b].long()[j // block_size] * block_size + j % block_size
+        kv = cache[rows].float()
+        k = kv[:, :nk].view(-1, kv_heads, dim).repeat_interleave(rep, 1)
+        v = kv[:, nk:].view(-1, kv_heads, vdim).repeat_interleave(rep, 1)
+        p = positions[a:e].long()[:, None]
+        dist = (p - j[None, :]).float()
+        s = torch.einsum("thd,jhd->htj", q[a:e].float(), k) * scale
+        s = s - sl * dist[None] + pos_bias.float()[:, None, None]
+        ok = j[None, :] <= p
+        if window > 0:
+            ok = ok & ((p - j[None, :] < window) | (j[None, :] < keep_first))
+        w = torch.sigmoid(s) * ok[None]
+        out[a:e] = torch.einsum("htj,jhd->thd", w, v)
+    return out.reshape(T, heads * vdim).to(out_dtype)
 
 
 def moe_route_all(h, router_w, correction, top, scale):

@@ -125,8 +125,10 @@ def test_latent_cache_write_and_rotation(dev):
     pos = torch.tensor([0, 1, 2, 40, 41, 1000], dtype=torch.int32)
     rows = torch.tensor([5, 0, 3, 9, 8, 1], dtype=torch.int32)
     cache = torch.zeros(12, r + rd, dtype=dtype, device=device)
-    q_rot = SM.latent_prepare(proj.to(device, dtype), H, dn, rd, r, True, nw.to(device), eps,
-                              pos.to(device), base, dims, rows.to(device), cache)
+    pj = proj.to(device, dtype)
+    q_rot = SM.latent_prepare(pj[:, :H * (dn + rd)], pj[:, H * (dn + rd):], H, dn, rd, r,
+                              nw.to(device), eps, pos.to(device), base, dims,
+                              rows.to(device), cache)
     for t in range(T):
         d = proj[t, H * (dn + rd):].double()
         c = O.norm_plain(d[:r], nw.double(), eps)
