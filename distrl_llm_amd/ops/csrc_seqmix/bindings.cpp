@@ -3,7 +3,7 @@
 #include <vector>
 
 std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
-                                          double eps, bool out_bf16);
+                                          double eps, bool out_bf16, double offset);
 void gated_residual_add(torch::Tensor x, torch::Tensor mix,
                         c10::optional<torch::Tensor> ff, torch::Tensor gates,
                         torch::Tensor gate_b, double mult);
@@ -14,19 +14,22 @@ std::vector<torch::Tensor> gated_residual_norm(
 torch::Tensor causal_tap_conv(torch::Tensor h, torch::Tensor w, torch::Tensor tails,
                               torch::Tensor cu, torch::Tensor tok_seq,
                               torch::Tensor slots, bool out_bf16);
-torch::Tensor latent_prepare(torch::Tensor proj, int64_t heads, int64_t dim,
-                             int64_t rot_dim, int64_t kv_rank, bool own_cache,
+torch::Tensor latent_prepare(torch::Tensor q, c10::optional<torch::Tensor> dkv, int64_t heads,
+                             int64_t dim, int64_t rot_dim, int64_t kv_rank,
                              c10::optional<torch::Tensor> norm_w, double eps,
                              torch::Tensor positions, double rope_base,
                              int64_t rope_dims, torch::Tensor page_slot,
-                             torch::Tensor cache);
+                             torch::Tensor cache, c10::optional<torch::Tensor> freqs,
+                             double mag, bool pairs);
 torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
                                       torch::Tensor cache, int64_t kv_rank,
                                       torch::Tensor block_tables, int64_t block_size,
                                       torch::Tensor tok_seq, torch::Tensor positions,
                                       int64_t window, double scale,
                                       c10::optional<torch::Tensor> tiles,
-                                      int64_t max_tile_queries);
+                                      int64_t max_tile_queries,
+                                      c10::optional<torch::Tensor> sink,
+                                      c10::optional<torch::Tensor> gate);
 torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor state,
                           torch::Tensor cu, torch::Tensor slots,
                           c10::optional<torch::Tensor> chunks,
@@ -46,8 +49,20 @@ torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tail
                             bool out_bf16);
 c10::optional<torch::Tensor> sandwich_residual_norm(
     torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2, torch::Tensor post_w,
-    c10::optional<torch::Tensor> next_w, double eps, bool out_bf16);
+    c10::optional<torch::Tensor> next_w, double eps, bool out_bf16, double offset,
+    double y_scale, double y2_scale, bool cast_next);
 torch::Tensor capped_glu(torch::Tensor gu, double limit);
+torch::Tensor silu_glu(torch::Tensor gu);
+torch::Tensor qk_norm_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
+                               int64_t vdim, torch::Tensor q_norm_w, torch::Tensor k_norm_w,
+                               double eps, torch::Tensor page_slot, torch::Tensor cache);
+torch::Tensor sigmoid_attention(torch::Tensor q, torch::Tensor cache, int64_t heads,
+                                int64_t kv_heads, int64_t dim, int64_t vdim,
+                                torch::Tensor block_tables, int64_t block_size,
+                                torch::Tensor tok_seq, torch::Tensor positions, double scale,
+                                int64_t window, int64_t keep_first, torch::Tensor slopes,
+                                torch::Tensor pos_bias, c10::optional<torch::Tensor> tiles,
+                                int64_t max_tile_queries);
 torch::Tensor rope_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
                             int64_t vdim, torch::Tensor positions, double rope_base,
                             int64_t rope_dims, torch::Tensor page_slot, torch::Tensor cache,
@@ -66,7 +81,8 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
                                c10::optional<torch::Tensor> ab_w, torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
                                double eps, torch::Tensor state, torch::Tensor cu,
                                torch::Tensor slots, int64_t heads, int64_t kv_heads,
-                               int64_t dim, int64_t vdim);
+                               int64_t dim, int64_t vdim,
+                               c10::optional<torch::Tensor> decay_up, bool gate_sigmoid);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("offset_rmsnorm", &offset_rmsnorm, "offset-weight RMS norm -> (fp32, dtype)");
@@ -87,6 +103,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sandwich_residual_norm", &sandwich_residual_norm,
         "closing norm + residual sum + next opening norm");
   m.def("capped_glu", &capped_glu, "clamped GLU activation");
+  m.def("silu_glu", &silu_glu, "SiLU-gated GLU activation");
+  m.def("qk_norm_kv_write", &qk_norm_kv_write, "per-head RMS norm of q/k, K/V cache write");
+  m.def("sigmoid_attention", &sigmoid_attention,
+        "paged GQA with sigmoid weights, distance penalty, window with kept first tokens");
   m.def("rope_kv_write", &rope_kv_write, "pair rotary on q/k, value blend, K/V cache write");
   m.def("sink_attention", &sink_attention,
         "paged GQA with capped scores, sinks and head mixing");

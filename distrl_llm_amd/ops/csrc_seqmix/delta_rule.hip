@@ -10,6 +10,9 @@
 //                   S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
 //                   inputs arrive in chunks through LDS, one chunk ahead
 //   delta_finish    per (token, head): o / rms(o) * norm_w * silu(gate)
+//                   (or * sigmoid(gate))
+// With a decay per head and key channel (delta_channel_decay forms it from a
+// low-rank input) the scan multiplies every state row by its own factor.
 // The scan is strictly sequential over a row's tokens, so a prompt cut into
 // portions gives bit-identical states and outputs.
 #include <torch/extension.h>
@@ -79,6 +82,35 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
   }
 }
 
+// Per-channel decays: ab row = [strength (H) | low-rank decay input (R)];
+// step = softplus(up[h dk + k] . input + dt_bias[h dk + k]),
+// decay[t, h, k] = exp(-exp(a_log[h]) step) for k < dk, 1 in the padding;
+// beta[t, h] = sigmoid(strength). One workgroup per token.
+__global__ __launch_bounds__(256) void delta_channel_decay_kernel(
+    const float* __restrict__ ab, int H, int R, const float* __restrict__ up,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, int dk, int dkp,
+    float* __restrict__ beta, float* __restrict__ decay) {
+  extern __shared__ float din[];                // R decay inputs of the token
+  const int64_t t = blockIdx.x;
+  const float* row = ab + t * (H + R);
+  for (int i = threadIdx.x; i < R; i += blockDim.x) din[i] = row[H + i];
+  for (int h = threadIdx.x; h < H; h += blockDim.x) beta[t * H + h] = sm_sigmoid(row[h]);
+  __syncthreads();
+  for (int i = threadIdx.x; i < H * dkp; i += blockDim.x) {
+    const int h = i / dkp, k = i % dkp;
+    float d = 1.0f;
+    if (k < dk) {
+      const float* w = up + (int64_t)(h * dk + k) * R;
+      float z = 0.f;
+      for (int j = 0; j < R; ++j) z = fmaf(w[j], din[j], z);
+      z += dt_bias[h * dk + k];
+      const float sp = (z > 20.f) ? z : log1pf(expf(z));
+      d = expf(-expf(a_log[h]) * sp);
+    }
+    decay[(t * H + h) * dkp + k] = d;
+  }
+}
+
 // One workgroup (4 waves) per (row, head, block of 256 / KS value columns).
 // Lane = (column, ks): it holds DR_ROWS state rows (8 or 32) of its column,
 // starting at ks * DR_ROWS (few rows per lane when there are few sequence
@@ -114,7 +146,9 @@ SM_INLINE float dr_column_sum(float x) {
   return x;
 }
 
-template <typename T, int KS, int DR_ROWS>
+// CH: the decay is a row of DKP factors per (token, head), staged beside the
+// token's k and q rows, instead of one factor per (token, head).
+template <typename T, int KS, int DR_ROWS, bool CH>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const T* __restrict__ qkv, int C, const float* __restrict__ qn,
     const float* __restrict__ kn, const float* __restrict__ beta,
@@ -124,8 +158,10 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   constexpr int COLS = 64 / KS;                 // columns per wave
   constexpr int DKP = KS * DR_ROWS;
   constexpr int ROW4 = DKP / 4;                 // float4 per q or k row
-  constexpr int NPRE = DR_CH * 2 * ROW4 / 256;  // float4 per thread and chunk
-  __shared__ float4 kq4[DR_CH * 2 * ROW4];      // [token][k | q][DKP]
+  constexpr int NR = CH ? 3 : 2;                // staged rows per token
+  constexpr int NSTAGE = DR_CH * NR * ROW4;
+  constexpr int NPRE = (NSTAGE + 255) / 256;    // float4 per thread and chunk
+  __shared__ float4 kq4[NSTAGE];                // [token][k | q (| decay)][DKP]
   __shared__ float sc[DR_CH * 2];               // [token][decay | beta]
   const int b = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -162,8 +198,11 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     #pragma unroll
     for (int j = 0; j < NPRE; ++j) {
       const int i = tid + 256 * j;
-      const int tok = i / (2 * ROW4), rem = i % (2 * ROW4);
-      const float* src = (rem >= ROW4 ? qn : kn) + ((int64_t)(tb + min(tok, n - 1)) * G + g) * DKP;
+      if (NSTAGE % 256 != 0 && i >= NSTAGE) break;
+      const int tok = i / (NR * ROW4), rem = i % (NR * ROW4);
+      const int64_t tt = tb + min(tok, n - 1);
+      const float* src = (rem >= 2 * ROW4) ? decay + (tt * H + h) * DKP
+                                           : (rem >= ROW4 ? qn : kn) + (tt * G + g) * DKP;
       pre[j] = reinterpret_cast<const float4*>(src)[rem % ROW4];
     }
     #pragma unroll
@@ -171,12 +210,13 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
       vout[i] = to_f(qkv[(int64_t)(tb + min(i, n - 1)) * C + voff]);
     if (tid < 2 * DR_CH) {
       const int64_t t = tb + min(tid >> 1, n - 1);
-      psc = (tid & 1) ? beta[t * H + h] : decay[t * H + h];
+      psc = (tid & 1) ? beta[t * H + h] : (CH ? 1.0f : decay[t * H + h]);
     }
   };
   auto stash = [&]() {
     #pragma unroll
-    for (int j = 0; j < NPRE; ++j) kq4[tid + 256 * j] = pre[j];
+    for (int j = 0; j < NPRE; ++j)
+      if (NSTAGE % 256 == 0 || tid + 256 * j < NSTAGE) kq4[tid + 256 * j] = pre[j];
     if (tid < 2 * DR_CH) sc[tid] = psc;
   };
 
@@ -190,7 +230,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     #pragma unroll
     for (int i = 0; i < DR_CH; ++i) {
       if (i >= n) break;
-      const float4* kp = kq4 + (i * 2) * ROW4 + ks * (DR_ROWS / 4);
+      const float4* kp = kq4 + (i * NR) * ROW4 + ks * (DR_ROWS / 4);
       const float4* qp = kp + ROW4;
       const float dec = sc[2 * i], bt = sc[2 * i + 1];
       float4 kk[DR_ROWS / 4];
@@ -198,7 +238,12 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
       #pragma unroll
       for (int r = 0; r < DR_ROWS; r += 4) {
         const float4 k4 = kk[r / 4] = kp[r / 4];
-        S[r] *= dec; S[r + 1] *= dec; S[r + 2] *= dec; S[r + 3] *= dec;
+        if (CH) {
+          const float4 d4 = kp[2 * ROW4 + r / 4];
+          S[r] *= d4.x; S[r + 1] *= d4.y; S[r + 2] *= d4.z; S[r + 3] *= d4.w;
+        } else {
+          S[r] *= dec; S[r + 1] *= dec; S[r + 2] *= dec; S[r + 3] *= dec;
+        }
         sk0 = fmaf(S[r], k4.x, sk0);
         sk1 = fmaf(S[r + 1], k4.y, sk1);
         sk0 = fmaf(S[r + 2], k4.z, sk0);
@@ -249,7 +294,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
 template <typename T>
 __global__ __launch_bounds__(64) void delta_finish_kernel(
     const float* __restrict__ o, const T* __restrict__ gate, int64_t ldg,
-    const float* __restrict__ norm_w, float eps, int H, int vd, T* __restrict__ out) {
+    const float* __restrict__ norm_w, float eps, int H, int vd, int gate_sigmoid,
+    T* __restrict__ out) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* src = o + (t * H + h) * vd;
@@ -259,17 +305,18 @@ __global__ __launch_bounds__(64) void delta_finish_kernel(
   const float inv = 1.0f / sqrtf(ss / (float)vd + eps);
   for (int d = lane; d < vd; d += 64) {
     const float gt = to_f(gate[t * ldg + h * vd + d]);
-    out[(t * H + h) * vd + d] = from_f<T>(src[d] * inv * norm_w[d] * (gt * sm_sigmoid(gt)));
+    const float act = gate_sigmoid ? sm_sigmoid(gt) : gt * sm_sigmoid(gt);
+    out[(t * H + h) * vd + d] = from_f<T>(src[d] * inv * norm_w[d] * act);
   }
 }
 
-template <typename T>
+template <typename T, bool CH>
 void launch_scan(int KS, int R, dim3 grid, hipStream_t stream, const T* qkv, int C, const float* qn,
                  const float* kn, const float* beta, const float* decay, float* state,
                  const int* cu, const int* slots, int H, int G, int dk, int vd, float* o) {
 #define DR_CASE(N, RR)                                                                        \
   if (KS == N && R == RR) {                                                                   \
-    delta_scan_kernel<T, N, RR><<<dim3(grid.x, grid.y, SM_CDIV(vd, 256 / N)), 256, 0, stream>>>( \
+    delta_scan_kernel<T, N, RR, CH><<<dim3(grid.x, grid.y, SM_CDIV(vd, 256 / N)), 256, 0, stream>>>( \
         qkv, C, qn, kn, beta, decay, state, cu, slots, H, G, dk, vd, o);                      \
     return;                                                                                   \
   }
@@ -288,7 +335,8 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
                                torch::Tensor a_log, torch::Tensor dt_bias, torch::Tensor onorm_w,
                                double eps, torch::Tensor state, torch::Tensor cu,
                                torch::Tensor slots, int64_t heads, int64_t kv_heads,
-                               int64_t dim, int64_t vdim) {
+                               int64_t dim, int64_t vdim,
+                               c10::optional<torch::Tensor> decay_up, bool gate_sigmoid) {
   SM_CHECK_CUDA(qkv);
   SM_CHECK_CUDA(a_log); SM_CHECK_F32(a_log); SM_CHECK_CUDA(dt_bias); SM_CHECK_F32(dt_bias);
   SM_CHECK_CUDA(onorm_w); SM_CHECK_F32(onorm_w); SM_CHECK_CUDA(state); SM_CHECK_F32(state);
@@ -303,6 +351,15 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
               gate.size(1) == H * vd && gate.scalar_type() == qkv.scalar_type(), "gated_delta_rule: gate layout");
   // the write strength / step inputs: given as [T, 2H] fp32, or computed here
   // from the mixer input h [T, D] and the fp32 matrix ab_w [2H, D]
+  const bool chan = decay_up.has_value();
+  const int Rk = chan ? (int)decay_up->size(1) : 0;       // low-rank decay inputs
+  const int abw = chan ? H + Rk : 2 * H;
+  if (chan) {
+    SM_CHECK_CUDA(*decay_up); SM_CHECK_F32(*decay_up);
+    TORCH_CHECK(decay_up->dim() == 2 && decay_up->size(0) == (int64_t)H * dk && Rk >= 1 &&
+                Rk <= 8192 && ab_opt.has_value(),
+                "gated_delta_rule: channel decays need decay_up [H dim, R] and ab [T, H + R]");
+  }
   const float* abp = nullptr;
   const float* abwp = nullptr;
   const void* hp = nullptr;
@@ -311,7 +368,7 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
   if (ab_opt.has_value()) {
     const torch::Tensor& ab = *ab_opt;
     SM_CHECK_CUDA(ab); SM_CHECK_F32(ab);
-    TORCH_CHECK(ab.dim() == 2 && ab.size(0) == T && ab.size(1) == 2 * H, "gated_delta_rule: ab is [T, 2H]");
+    TORCH_CHECK(ab.dim() == 2 && ab.size(0) == T && ab.size(1) == abw, "gated_delta_rule: ab width");
     abp = ab.data_ptr<float>();
   } else {
     TORCH_CHECK(h_opt.has_value() && ab_w_opt.has_value(), "gated_delta_rule: ab, or h with ab_w");
@@ -326,7 +383,8 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
     Dh = hh.size(1);
     abwp = w.data_ptr<float>();
   }
-  TORCH_CHECK(a_log.numel() == H && dt_bias.numel() == H && onorm_w.numel() == vd, "gated_delta_rule: per-head tensors");
+  TORCH_CHECK(a_log.numel() == H && dt_bias.numel() == (chan ? (int64_t)H * dk : H) &&
+              onorm_w.numel() == vd, "gated_delta_rule: per-head tensors");
   TORCH_CHECK(state.dim() == 2 && state.size(1) == (int64_t)H * dk * vd && cu.numel() == B + 1,
               "gated_delta_rule: state/batch layout");
   TORCH_CHECK(dk <= 256, "gated_delta_rule: key dim above 256");
@@ -345,41 +403,62 @@ torch::Tensor gated_delta_rule(torch::Tensor qkv, torch::Tensor gate,
   if (T == 0 || B == 0) return out;
   auto f32 = qkv.options().dtype(at::kFloat);
   auto qn = torch::empty({T, G, dkp}, f32), kn = torch::empty({T, G, dkp}, f32);
-  auto beta = torch::empty({T, H}, f32), decay = torch::empty({T, H}, f32);
+  auto beta = torch::empty({T, H}, f32);
+  auto decay = chan ? torch::empty({T, H, dkp}, f32) : torch::empty({T, H}, f32);
   auto o = torch::empty({T, H, vd}, f32);
   auto stream = at::cuda::getCurrentCUDAStream();
   const bool bf16 = qkv.scalar_type() == at::kBFloat16;
   if (!bf16) SM_CHECK_F32(qkv);
   dim3 gscan(B, H), gfin(T, H);
   dim3 gprep(T, abp != nullptr ? 1 : 1 + SM_CDIV(2 * H, 4));
+  // channel decays: the unit q/k rows come from delta_prepare (which then
+  // leaves beta/decay alone), strengths and decays from their own kernel
+  const float* abq = chan ? nullptr : abp;
+  if (chan) {
+    delta_channel_decay_kernel<<<T, 256, Rk * sizeof(float), stream>>>(
+        abp, H, Rk, decay_up->data_ptr<float>(), a_log.data_ptr<float>(),
+        dt_bias.data_ptr<float>(), dk, dkp, beta.data_ptr<float>(), decay.data_ptr<float>());
+    SM_CHECK_LAUNCH();
+  }
   if (bf16) {
     const bf16_t* xp = reinterpret_cast<const bf16_t*>(qkv.data_ptr());
     delta_prepare_kernel<bf16_t><<<gprep, 256, 0, stream>>>(
-        xp, C, abp, reinterpret_cast<const bf16_t*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
+        xp, C, abq, reinterpret_cast<const bf16_t*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
         dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
-    launch_scan<bf16_t>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+    if (chan)
+      launch_scan<bf16_t, true>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+                        beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
+                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
+    else
+      launch_scan<bf16_t, false>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                         beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
                         cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();
     delta_finish_kernel<bf16_t><<<gfin, 64, 0, stream>>>(
         o.data_ptr<float>(), reinterpret_cast<const bf16_t*>(gate.data_ptr()), gate.stride(0),
-        onorm_w.data_ptr<float>(), (float)eps, H, vd, reinterpret_cast<bf16_t*>(out.data_ptr()));
+        onorm_w.data_ptr<float>(), (float)eps, H, vd, gate_sigmoid ? 1 : 0,
+        reinterpret_cast<bf16_t*>(out.data_ptr()));
   } else {
     const float* xp = qkv.data_ptr<float>();
     delta_prepare_kernel<float><<<gprep, 256, 0, stream>>>(
-        xp, C, abp, reinterpret_cast<const float*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
+        xp, C, abq, reinterpret_cast<const float*>(hp), ldh, abwp, Dh, a_log.data_ptr<float>(),
         dt_bias.data_ptr<float>(), H, G, dk, dkp,
         qn.data_ptr<float>(), kn.data_ptr<float>(), beta.data_ptr<float>(), decay.data_ptr<float>());
     SM_CHECK_LAUNCH();
-    launch_scan<float>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+    if (chan)
+      launch_scan<float, true>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
+                       beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
+                       cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
+    else
+      launch_scan<float, false>(KS, R, gscan, stream, xp, C, qn.data_ptr<float>(), kn.data_ptr<float>(),
                        beta.data_ptr<float>(), decay.data_ptr<float>(), state.data_ptr<float>(),
                        cu.data_ptr<int>(), slots.data_ptr<int>(), H, G, dk, vd, o.data_ptr<float>());
     SM_CHECK_LAUNCH();
     delta_finish_kernel<float><<<gfin, 64, 0, stream>>>(
         o.data_ptr<float>(), gate.data_ptr<float>(), gate.stride(0), onorm_w.data_ptr<float>(),
-        (float)eps, H, vd, out.data_ptr<float>());
+        (float)eps, H, vd, gate_sigmoid ? 1 : 0, out.data_ptr<float>());
   }
   SM_CHECK_LAUNCH();
   return out;

@@ -15,42 +15,54 @@
 
 namespace {
 
-// angle of pair i at position p: p * base^(-2 i / dims), all fp32
-SM_INLINE void rot_cs(int p, int i, float base, int dims, float* c, float* s) {
-  const float f = powf(base, -2.0f * (float)i / (float)dims);
+// angle of pair i at position p: p * base^(-2 i / dims), or p * freqs[i] with
+// cos and sin scaled by mag when a frequency table is given; all fp32
+SM_INLINE void rot_cs(int p, int i, float base, int dims, const float* freqs, float mag,
+                      float* c, float* s) {
+  const float f = freqs != nullptr ? freqs[i] : powf(base, -2.0f * (float)i / (float)dims);
   sincosf((float)p * f, s, c);
+  if (freqs != nullptr) { *c *= mag; *s *= mag; }
 }
 
-// One workgroup per token. proj row = [q (H * (dn + rd)) | d (r + rd)].
+// Entry k of a rotated vector v (first dims entries rotated): pairs
+// (i, i + dims/2), or (2i, 2i+1) with PAIRS.
+template <typename T>
+SM_INLINE float rot_entry(const T* v, int k, int p, float base, int dims, const float* freqs,
+                          float mag, bool pairs) {
+  if (k >= dims) return to_f(v[k]);
+  const int half = dims / 2;
+  int pi, ia, ib;
+  bool first;
+  if (pairs) { pi = k >> 1; ia = 2 * pi; ib = ia + 1; first = (k & 1) == 0; }
+  else { pi = (k < half) ? k : k - half; ia = pi; ib = pi + half; first = k < half; }
+  float c, s;
+  rot_cs(p, pi, base, dims, freqs, mag, &c, &s);
+  const float a = to_f(v[ia]), b = to_f(v[ib]);
+  return first ? a * c - b * s : b * c + a * s;
+}
+
+// One workgroup per token. q row = H * (dn + rd) query entries, d row (when
+// the layer owns a cache) = [latent (r) | shared key part (rd)]; rows are
+// ldq / ldd apart.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(
-    const T* __restrict__ proj, int P, int H, int dn, int rd, int r, int own,
-    const float* __restrict__ norm_w, float eps, const int* __restrict__ positions,
-    float base, int dims, const int* __restrict__ page_slot, T* __restrict__ cache,
+    const T* __restrict__ q, int64_t ldq, const T* __restrict__ dkv, int64_t ldd, int H,
+    int dn, int rd, int r, const float* __restrict__ norm_w, float eps,
+    const int* __restrict__ positions, float base, int dims, const float* __restrict__ freqs,
+    float mag, int pairs, const int* __restrict__ page_slot, T* __restrict__ cache,
     float* __restrict__ q_rot) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
-  const T* row = proj + t * P;
+  const T* row = q + t * ldq;
   const int p = positions[t];
-  const int half = dims / 2;
   // rotated query part of every head
   for (int i = threadIdx.x; i < H * rd; i += blockDim.x) {
     const int hd = i / rd, k = i % rd;
-    const T* qr = row + hd * (dn + rd) + dn;
-    float v;
-    if (k < dims) {
-      const int pi = (k < half) ? k : k - half;
-      float c, s;
-      rot_cs(p, pi, base, dims, &c, &s);
-      const float a = to_f(qr[pi]), b = to_f(qr[pi + half]);
-      v = (k < half) ? a * c - b * s : b * c + a * s;
-    } else {
-      v = to_f(qr[k]);
-    }
-    q_rot[(t * H + hd) * rd + k] = v;
+    q_rot[(t * H + hd) * rd + k] =
+        rot_entry(row + hd * (dn + rd) + dn, k, p, base, dims, freqs, mag, pairs != 0);
   }
-  if (!own) return;
-  const T* d = row + H * (dn + rd);
+  if (dkv == nullptr) return;
+  const T* d = dkv + t * ldd;
   float ss = 0.f;
   for (int k = threadIdx.x; k < r; k += blockDim.x) {
     const float v = to_f(d[k]);
@@ -61,19 +73,20 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   T* dst = cache + (int64_t)page_slot[t] * (r + rd);
   for (int k = threadIdx.x; k < r; k += blockDim.x)
     dst[k] = from_f<T>(to_f(d[k]) * inv * norm_w[k]);
-  for (int k = threadIdx.x; k < rd; k += blockDim.x) {
-    float v;
-    if (k < dims) {
-      const int pi = (k < half) ? k : k - half;
-      float c, s;
-      rot_cs(p, pi, base, dims, &c, &s);
-      const float a = to_f(d[r + pi]), b = to_f(d[r + pi + half]);
-      v = (k < half) ? a * c - b * s : b * c + a * s;
-    } else {
-      v = to_f(d[r + k]);
-    }
-    dst[r + k] = from_f<T>(v);
-  }
+  for (int k = threadIdx.x; k < rd; k += blockDim.x)
+    dst[r + k] = from_f<T>(rot_entry(d + r, k, p, base, dims, freqs, mag, pairs != 0));
+}
+
+// Closing factor of one (token, head): 1 / (sum + e^(sink - max)) when the
+// head has a sink term in its softmax denominator, times sigmoid(gate) when
+// the head's result is gated.
+template <typename T>
+SM_INLINE float lat_close(float M, float L, const float* sink, const T* gate, int64_t ldg,
+                          int64_t t, int hd) {
+  if (sink != nullptr) L += expf(sink[hd] - M);
+  float f = 1.0f / L;
+  if (gate != nullptr) f *= sm_sigmoid(to_f(gate[t * ldg + hd]));
+  return f;
 }
 
 // One wave per (token, head). Keys lo..p of the token's sequence are taken
@@ -89,6 +102,7 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
     const int* __restrict__ block_tables, int max_nb, int block_size,
     const int* __restrict__ tok_seq, const int* __restrict__ positions,
     int Tn, int H, int r, int rd, int window, float scale,
+    const float* __restrict__ sink, const T* __restrict__ gate, int64_t ldg,
     T* __restrict__ out) {            // [H, Tn, r]
   extern __shared__ float lds[];
   float* q = lds;                       // r + rd
@@ -138,7 +152,7 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
       }
     }
   }
-  const float invl = 1.0f / l;
+  const float invl = lat_close(m, l, sink, gate, ldg, t, hd);
   #pragma unroll
   for (int i = 0; i < SM_LAT_REGS; ++i) {
     const int k = lane + 64 * i;
@@ -186,7 +200,8 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
     const int* __restrict__ tiles,      // [ntiles, 3] = (batch row, first token, queries)
     const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
     float scale, int nq_cap, bf16_t* __restrict__ out,
-    int ksplit, float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    int ksplit, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const float* __restrict__ sink, const bf16_t* __restrict__ gate, int64_t ldg) {
   // ksplit > 1 (HEADS only): blockIdx.z takes a contiguous share of the key
   // blocks and leaves (max, sum, unnormalised latent sum) for the combine
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -395,8 +410,8 @@ __global__ __launch_bounds__(256) void latent_attention_tiled_kernel(
         const float mw = ml[(w * LT_TQ + q) * 2];
         if (mw != -INFINITY) L += ml[(w * LT_TQ + q) * 2 + 1] * expf(mw - M);
       }
-      const float invL = 1.0f / L;
       const int tq_ = HEADS ? t0 : t0 + q, hq_ = HEADS ? hd + q : hd;
+      const float invL = lat_close(M, L, sink, gate, ldg, tq_, hq_);
       if (ksplit > 1 && l == 0) {
         part_ml[(((int64_t)tq_ * H + hq_) * ksplit + blockIdx.z) * 2] = M;
         part_ml[(((int64_t)tq_ * H + hq_) * ksplit + blockIdx.z) * 2 + 1] = L;
@@ -446,7 +461,8 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
     int max_nb, int block_size, const int* __restrict__ tiles,
     const int* __restrict__ positions, int Tn, int H, int r, int rd, int window,
     float scale, bf16_t* __restrict__ out, int ksplit,
-    float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const float* __restrict__ sink, const bf16_t* __restrict__ gate, int64_t ldg) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int W = r + rd;
   const int Wp = LC_ROW(W);
@@ -620,6 +636,15 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
       }
     }
   }
+  float fin[4];
+  #pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    const int q = lk * 4 + rr;
+    fin[rr] = 0.f;
+    if (q < nq && ksplit <= 1)
+      fin[rr] = lat_close(m[rr], lsum[rr], sink, gate, ldg, HEADS ? t0 : t0 + q,
+                          HEADS ? hd + q : hd);
+  }
   #pragma unroll
   for (int i = 0; i < LC_NT; ++i) {
     const int nt = wave + 4 * i;
@@ -633,7 +658,7 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
           if (ksplit > 1)
             part_acc[(((int64_t)tq * H + hq) * ksplit + blockIdx.z) * r + f] = acc[i][rr];
           else
-            out[((int64_t)hq * Tn + tq) * r + f] = __float2bfloat16(acc[i][rr] / lsum[rr]);
+            out[((int64_t)hq * Tn + tq) * r + f] = __float2bfloat16(acc[i][rr] * fin[rr]);
         }
       }
     }
@@ -643,7 +668,8 @@ __global__ __launch_bounds__(256) void latent_attention_coop_kernel(
 // Merge the key splits of one (token, head): out = sum_z acc_z e^(m_z - M) / L.
 __global__ __launch_bounds__(256) void latent_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    int Tn, int H, int r, int ksplit, bf16_t* __restrict__ out) {
+    int Tn, int H, int r, int ksplit, bf16_t* __restrict__ out,
+    const float* __restrict__ sink, const bf16_t* __restrict__ gate, int64_t ldg) {
   const int t = blockIdx.x / H, hd = blockIdx.x % H;
   const float* ml = part_ml + (int64_t)blockIdx.x * ksplit * 2;
   float M = -INFINITY;
@@ -651,7 +677,7 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(
   float L = 0.f;
   for (int z = 0; z < ksplit; ++z)
     if (ml[z * 2] != -INFINITY) L += ml[z * 2 + 1] * expf(ml[z * 2] - M);
-  const float invL = 1.0f / L;
+  const float invL = lat_close(M, L, sink, gate, ldg, t, hd);
   for (int f = threadIdx.x; f < r; f += blockDim.x) {
     float a = 0.f;
     for (int z = 0; z < ksplit; ++z)
@@ -663,44 +689,62 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(
 
 }  // namespace
 
-torch::Tensor latent_prepare(torch::Tensor proj, int64_t heads, int64_t dim,
-                             int64_t rot_dim, int64_t kv_rank, bool own_cache,
+torch::Tensor latent_prepare(torch::Tensor q, c10::optional<torch::Tensor> dkv, int64_t heads,
+                             int64_t dim, int64_t rot_dim, int64_t kv_rank,
                              c10::optional<torch::Tensor> norm_w, double eps,
                              torch::Tensor positions, double rope_base,
                              int64_t rope_dims, torch::Tensor page_slot,
-                             torch::Tensor cache) {
-  SM_CHECK_CUDA(proj); SM_CHECK_CUDA(positions); SM_CHECK_I32(positions);
+                             torch::Tensor cache, c10::optional<torch::Tensor> freqs,
+                             double mag, bool pairs) {
+  SM_CHECK_CUDA(positions); SM_CHECK_I32(positions);
   SM_CHECK_CUDA(page_slot); SM_CHECK_I32(page_slot); SM_CHECK_CUDA(cache);
-  const int64_t T = proj.size(0);
-  const int P = proj.size(1);
+  const int64_t T = q.size(0);
   const int64_t qs = heads * (dim + rot_dim);
-  TORCH_CHECK(P == qs + (own_cache ? kv_rank + rot_dim : 0), "latent_prepare: projection width");
+  TORCH_CHECK(q.is_cuda() && q.dim() == 2 && q.stride(1) == 1 && q.size(1) == qs,
+              "latent_prepare: query rows");
   TORCH_CHECK(rope_dims % 2 == 0 && rope_dims <= rot_dim, "latent_prepare: rope dims");
   TORCH_CHECK(positions.numel() == T && page_slot.numel() == T, "latent_prepare: batch layout");
   TORCH_CHECK(cache.dim() == 2 && cache.size(1) == kv_rank + rot_dim &&
-              cache.scalar_type() == proj.scalar_type(), "latent_prepare: cache shape/dtype");
+              cache.scalar_type() == q.scalar_type(), "latent_prepare: cache shape/dtype");
   const float* nw = nullptr;
-  if (own_cache) {
+  const void* dp = nullptr;
+  int64_t ldd = 0;
+  if (dkv.has_value()) {
+    TORCH_CHECK(dkv->is_cuda() && dkv->dim() == 2 && dkv->stride(1) == 1 && dkv->size(0) == T &&
+                dkv->size(1) == kv_rank + rot_dim && dkv->scalar_type() == q.scalar_type(),
+                "latent_prepare: latent rows");
     TORCH_CHECK(norm_w.has_value(), "latent_prepare: norm weight missing");
     SM_CHECK_CUDA(*norm_w); SM_CHECK_F32(*norm_w);
     TORCH_CHECK(norm_w->numel() == kv_rank, "latent_prepare: norm weight size");
     nw = norm_w->data_ptr<float>();
+    dp = dkv->data_ptr();
+    ldd = dkv->stride(0);
   }
-  auto q_rot = torch::empty({T, heads, rot_dim}, proj.options().dtype(at::kFloat));
+  const float* fp = nullptr;
+  if (freqs.has_value()) {
+    SM_CHECK_CUDA(*freqs); SM_CHECK_F32(*freqs);
+    TORCH_CHECK(freqs->numel() == rope_dims / 2, "latent_prepare: one frequency per pair");
+    fp = freqs->data_ptr<float>();
+  } else {
+    TORCH_CHECK(!pairs && mag == 1.0, "latent_prepare: pair layout and scaling need a frequency table");
+  }
+  auto q_rot = torch::empty({T, heads, rot_dim}, q.options().dtype(at::kFloat));
   if (T == 0) return q_rot;
   auto stream = at::cuda::getCurrentCUDAStream();
-  if (proj.scalar_type() == at::kBFloat16)
+  if (q.scalar_type() == at::kBFloat16)
     latent_prepare_kernel<bf16_t><<<T, 256, 0, stream>>>(
-        reinterpret_cast<const bf16_t*>(proj.data_ptr()), P, heads, dim, rot_dim, kv_rank,
-        own_cache ? 1 : 0, nw, (float)eps, positions.data_ptr<int>(), (float)rope_base,
-        (int)rope_dims, page_slot.data_ptr<int>(), reinterpret_cast<bf16_t*>(cache.data_ptr()),
+        reinterpret_cast<const bf16_t*>(q.data_ptr()), q.stride(0),
+        reinterpret_cast<const bf16_t*>(dp), ldd, heads, dim, rot_dim, kv_rank, nw, (float)eps,
+        positions.data_ptr<int>(), (float)rope_base, (int)rope_dims, fp, (float)mag, pairs ? 1 : 0,
+        page_slot.data_ptr<int>(), reinterpret_cast<bf16_t*>(cache.data_ptr()),
         q_rot.data_ptr<float>());
   else {
-    SM_CHECK_F32(proj);
+    SM_CHECK_F32(q);
     latent_prepare_kernel<float><<<T, 256, 0, stream>>>(
-        proj.data_ptr<float>(), P, heads, dim, rot_dim, kv_rank, own_cache ? 1 : 0, nw,
-        (float)eps, positions.data_ptr<int>(), (float)rope_base, (int)rope_dims,
-        page_slot.data_ptr<int>(), cache.data_ptr<float>(), q_rot.data_ptr<float>());
+        q.data_ptr<float>(), q.stride(0), reinterpret_cast<const float*>(dp), ldd, heads, dim,
+        rot_dim, kv_rank, nw, (float)eps, positions.data_ptr<int>(), (float)rope_base,
+        (int)rope_dims, fp, (float)mag, pairs ? 1 : 0, page_slot.data_ptr<int>(),
+        cache.data_ptr<float>(), q_rot.data_ptr<float>());
   }
   SM_CHECK_LAUNCH();
   return q_rot;
@@ -712,7 +756,9 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
                                       torch::Tensor tok_seq, torch::Tensor positions,
                                       int64_t window, double scale,
                                       c10::optional<torch::Tensor> tiles,
-                                      int64_t max_tile_queries) {
+                                      int64_t max_tile_queries,
+                                      c10::optional<torch::Tensor> sink,
+                                      c10::optional<torch::Tensor> gate) {
   SM_CHECK_CUDA(q_lat); SM_CHECK_CUDA(q_rot); SM_CHECK_F32(q_rot); SM_CHECK_CUDA(cache);
   SM_CHECK_CUDA(block_tables); SM_CHECK_I32(block_tables);
   SM_CHECK_CUDA(tok_seq); SM_CHECK_I32(tok_seq); SM_CHECK_CUDA(positions); SM_CHECK_I32(positions);
@@ -726,6 +772,22 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
   TORCH_CHECK(cache.size(1) == r + rd && cache.scalar_type() == q_lat.scalar_type(),
               "latent attention: cache shape/dtype");
   TORCH_CHECK(tok_seq.numel() == T && positions.numel() == T && block_size > 0, "latent attention: batch layout");
+  const float* sinkp = nullptr;
+  const void* gatep = nullptr;
+  int64_t ldg = 0;
+  if (sink.has_value()) {
+    SM_CHECK_CUDA(*sink); SM_CHECK_F32(*sink);
+    TORCH_CHECK(sink->numel() == H, "latent attention: one sink per head");
+    sinkp = sink->data_ptr<float>();
+  }
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->dim() == 2 && gate->stride(1) == 1 && gate->size(0) == T &&
+                gate->size(1) == H && gate->scalar_type() == q_lat.scalar_type(),
+                "latent attention: gate is [T, H] in the model dtype");
+    gatep = gate->data_ptr();
+    ldg = gate->stride(0);
+  }
+  const bf16_t* gateb = reinterpret_cast<const bf16_t*>(gatep);
   auto out = torch::empty_like(q_lat);
   if (T == 0) return out;
   auto stream = at::cuda::getCurrentCUDAStream();
@@ -758,7 +820,7 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
             reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
             (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),
             positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
-            reinterpret_cast<bf16_t*>(out.data_ptr()), 1, nullptr, nullptr);
+            reinterpret_cast<bf16_t*>(out.data_ptr()), 1, nullptr, nullptr, sinkp, gateb, ldg);
         SM_CHECK_LAUNCH();
         return out;
       }
@@ -792,11 +854,12 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
             reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
             (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),
             positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
-            reinterpret_cast<bf16_t*>(out.data_ptr()), ks, pap, pmp);
+            reinterpret_cast<bf16_t*>(out.data_ptr()), ks, pap, pmp, sinkp, gateb, ldg);
         SM_CHECK_LAUNCH();
         if (ks > 1) {
           latent_combine_kernel<<<(int)(T * H), 256, 0, stream>>>(
-              pap, pmp, (int)T, H, r, ks, reinterpret_cast<bf16_t*>(out.data_ptr()));
+              pap, pmp, (int)T, H, r, ks, reinterpret_cast<bf16_t*>(out.data_ptr()), sinkp, gateb,
+              ldg);
           SM_CHECK_LAUNCH();
         }
         return out;
@@ -839,7 +902,7 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
           reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(), \
           (int)block_tables.size(1), (int)block_size, tiles->data_ptr<int>(),            \
           positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale, nq_cap, \
-          reinterpret_cast<bf16_t*>(out.data_ptr()), ksplit, pacc, pml);                \
+          reinterpret_cast<bf16_t*>(out.data_ptr()), ksplit, pacc, pml, sinkp, gateb, ldg); \
       } while (0)
     if (heads) {
       if (r <= 128) LT_LAUNCH(2, true);
@@ -854,7 +917,8 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
     if (ksplit > 1) {
       SM_CHECK_LAUNCH();
       latent_combine_kernel<<<(int)(T * H), 256, 0, stream>>>(
-          pacc, pml, (int)T, H, r, ksplit, reinterpret_cast<bf16_t*>(out.data_ptr()));
+          pacc, pml, (int)T, H, r, ksplit, reinterpret_cast<bf16_t*>(out.data_ptr()), sinkp, gateb,
+          ldg);
     }
     SM_CHECK_LAUNCH();
     return out;
@@ -865,7 +929,7 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
         reinterpret_cast<const bf16_t*>(q_lat.data_ptr()), q_rot.data_ptr<float>(),
         reinterpret_cast<const bf16_t*>(cache.data_ptr()), block_tables.data_ptr<int>(),
         (int)block_tables.size(1), (int)block_size, tok_seq.data_ptr<int>(),
-        positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale,
+        positions.data_ptr<int>(), (int)T, H, r, rd, (int)window, (float)scale, sinkp, gateb, ldg,
         reinterpret_cast<bf16_t*>(out.data_ptr()));
   else {
     SM_CHECK_F32(q_lat);
@@ -873,7 +937,8 @@ torch::Tensor latent_window_attention(torch::Tensor q_lat, torch::Tensor q_rot,
         q_lat.data_ptr<float>(), q_rot.data_ptr<float>(), cache.data_ptr<float>(),
         block_tables.data_ptr<int>(), (int)block_tables.size(1), (int)block_size,
         tok_seq.data_ptr<int>(), positions.data_ptr<int>(), (int)T, H, r, rd,
-        (int)window, (float)scale, out.data_ptr<float>());
+        (int)window, (float)scale, sinkp, reinterpret_cast<const float*>(gatep), ldg,
+        out.data_ptr<float>());
   }
   SM_CHECK_LAUNCH();
   return out;

@@ -10,14 +10,15 @@
 
 namespace {
 
-// h = x / sqrt(mean(x^2) + eps) * (1 + w); written as fp32 and (if hb) as T.
+// h = x / sqrt(mean(x^2) + eps) * (offset + w); written as fp32 and (if hb)
+// as T. Input rows are ldx apart (a column slice of a wider matrix).
 template <typename Tin, typename T>
 __global__ __launch_bounds__(256) void offset_rmsnorm_kernel(
-    const Tin* __restrict__ x, const float* __restrict__ w, float eps, int D,
-    float* __restrict__ h32, T* __restrict__ hb) {
+    const Tin* __restrict__ x, int64_t ldx, const float* __restrict__ w, float eps,
+    float offset, int D, float* __restrict__ h32, T* __restrict__ hb) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
-  const Tin* xr = x + row * D;
+  const Tin* xr = x + row * ldx;
   float ss = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     const float v = to_f(xr[d]);
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(256) void offset_rmsnorm_kernel(
   ss = sm_block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float v = to_f(xr[d]) * inv * (1.0f + w[d]);
+    const float v = to_f(xr[d]) * inv * (offset + w[d]);
     h32[row * D + d] = v;
     if (hb != nullptr) hb[row * D + d] = from_f<T>(v);
   }
@@ -152,51 +153,57 @@ template <typename T>
 __global__ __launch_bounds__(256) void sandwich_residual_kernel(
     float* __restrict__ x, const void* __restrict__ y, bool y_bf16,
     const void* __restrict__ y2, bool y2_bf16, const float* __restrict__ post_w,
-    const float* __restrict__ next_w, float eps, int D, T* __restrict__ h) {
+    const float* __restrict__ next_w, float eps, float offset, float ys, float y2s,
+    int D, T* __restrict__ h) {
+  // the closing norm is over s = ys * y (+ y2s * y2); h (when given) gets the
+  // next norm of the new row, or, without next_w, the new row itself
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   float ss = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float s = ld_any(y, y_bf16, row * D + d);
-    if (y2 != nullptr) s += ld_any(y2, y2_bf16, row * D + d);
+    float s = ys * ld_any(y, y_bf16, row * D + d);
+    if (y2 != nullptr) s += y2s * ld_any(y2, y2_bf16, row * D + d);
     ss += s * s;
   }
   ss = sm_block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   float xx = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float s = ld_any(y, y_bf16, row * D + d);
-    if (y2 != nullptr) s += ld_any(y2, y2_bf16, row * D + d);
-    const float v = x[row * D + d] + s * inv * (1.0f + post_w[d]);
+    float s = ys * ld_any(y, y_bf16, row * D + d);
+    if (y2 != nullptr) s += y2s * ld_any(y2, y2_bf16, row * D + d);
+    const float v = x[row * D + d] + s * inv * (offset + post_w[d]);
     x[row * D + d] = v;
     xx += v * v;
+    if (next_w == nullptr && h != nullptr) h[row * D + d] = from_f<T>(v);
   }
   if (next_w == nullptr) return;
   xx = sm_block_sum(xx, red);   // also orders the row's writes before the re-read
   const float inv2 = 1.0f / sqrtf(xx / (float)D + eps);
   for (int d = threadIdx.x; d < D; d += blockDim.x)
-    h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (1.0f + next_w[d]));
+    h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (offset + next_w[d]));
 }
 
 // gu rows = [gate (ff) | up (ff)]: g = min(gate, limit), u = clamp(up, +-limit),
-// out = g * sigmoid(1.702 g) * (u + 1).
-template <typename T>
+// out = g * sigmoid(1.702 g) * (u + 1); SILU: out = gate * sigmoid(gate) * up.
+template <typename T, bool SILU>
 __global__ __launch_bounds__(256) void capped_glu_kernel(
     const T* __restrict__ gu, int64_t n, int ff, float limit, T* __restrict__ out) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= n) return;
   const int64_t t = id / ff;
   const int f = id % ff;
-  out[id] = from_f<T>(sm_capped_glu(to_f(gu[t * 2 * ff + f]),
-                                    to_f(gu[t * 2 * ff + ff + f]), limit));
+  const float g = to_f(gu[t * 2 * ff + f]), u = to_f(gu[t * 2 * ff + ff + f]);
+  out[id] = from_f<T>(SILU ? g * sm_sigmoid(g) * u : sm_capped_glu(g, u, limit));
 }
 
 }  // namespace
 
 std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
-                                          double eps, bool out_bf16) {
-  SM_CHECK_CUDA(x); SM_CHECK_CUDA(w); SM_CHECK_F32(w);
-  TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1), "offset_rmsnorm: shapes");
+                                          double eps, bool out_bf16, double offset) {
+  SM_CHECK_CUDA(w); SM_CHECK_F32(w);
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1 && w.numel() == x.size(1),
+              "offset_rmsnorm: shapes");
+  const int64_t ldx = x.stride(0);
   const int64_t T = x.size(0);
   const int D = x.size(1);
   auto h32 = torch::empty({T, D}, x.options().dtype(at::kFloat));
@@ -206,12 +213,12 @@ std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
   bf16_t* hbp = out_bf16 ? reinterpret_cast<bf16_t*>(hb.data_ptr()) : nullptr;
   if (x.scalar_type() == at::kBFloat16) {
     offset_rmsnorm_kernel<bf16_t, bf16_t><<<T, 256, 0, stream>>>(
-        reinterpret_cast<const bf16_t*>(x.data_ptr()), w.data_ptr<float>(),
-        (float)eps, D, h32.data_ptr<float>(), hbp);
+        reinterpret_cast<const bf16_t*>(x.data_ptr()), ldx, w.data_ptr<float>(),
+        (float)eps, (float)offset, D, h32.data_ptr<float>(), hbp);
   } else {
     SM_CHECK_F32(x);
     offset_rmsnorm_kernel<float, bf16_t><<<T, 256, 0, stream>>>(
-        x.data_ptr<float>(), w.data_ptr<float>(), (float)eps, D,
+        x.data_ptr<float>(), ldx, w.data_ptr<float>(), (float)eps, (float)offset, D,
         h32.data_ptr<float>(), hbp);
   }
   SM_CHECK_LAUNCH();
@@ -379,7 +386,7 @@ torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tail
 c10::optional<torch::Tensor> sandwich_residual_norm(
     torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2,
     torch::Tensor post_w, c10::optional<torch::Tensor> next_w, double eps,
-    bool out_bf16) {
+    bool out_bf16, double offset, double y_scale, double y2_scale, bool cast_next) {
   SM_CHECK_CUDA(x); SM_CHECK_F32(x); SM_CHECK_CUDA(y); SM_CHECK_CUDA(post_w); SM_CHECK_F32(post_w);
   const int64_t T = x.size(0);
   const int D = x.size(1);
@@ -406,24 +413,30 @@ c10::optional<torch::Tensor> sandwich_residual_norm(
     TORCH_CHECK(next_w->numel() == D, "sandwich_residual_norm: norm weight");
     nw = next_w->data_ptr<float>();
     h = torch::empty({T, D}, x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  } else if (cast_next) {
+    TORCH_CHECK(out_bf16, "sandwich_residual_norm: a copy of the residual is made in bf16 only");
+    h = torch::empty({T, D}, x.options().dtype(at::kBFloat16));
   }
   if (T == 0) return h;
   auto stream = at::cuda::getCurrentCUDAStream();
   if (out_bf16)
     sandwich_residual_kernel<bf16_t><<<T, 256, 0, stream>>>(
-        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps, D,
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps,
+        (float)offset, (float)y_scale, (float)y2_scale, D,
         h.has_value() ? reinterpret_cast<bf16_t*>(h->data_ptr()) : nullptr);
   else
     sandwich_residual_kernel<float><<<T, 256, 0, stream>>>(
-        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps, D,
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps,
+        (float)offset, (float)y_scale, (float)y2_scale, D,
         h.has_value() ? h->data_ptr<float>() : nullptr);
   SM_CHECK_LAUNCH();
   return h;
 }
 
-torch::Tensor capped_glu(torch::Tensor gu, double limit) {
+template <bool SILU>
+static torch::Tensor glu_impl(torch::Tensor gu, double limit) {
   SM_CHECK_CUDA(gu);
-  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0, "capped_glu: rows are [gate | up]");
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0, "glu: rows are [gate | up]");
   const int64_t T = gu.size(0);
   const int ff = gu.size(1) / 2;
   auto out = torch::empty({T, ff}, gu.options());
@@ -431,14 +444,17 @@ torch::Tensor capped_glu(torch::Tensor gu, double limit) {
   if (n == 0) return out;
   auto stream = at::cuda::getCurrentCUDAStream();
   if (gu.scalar_type() == at::kBFloat16)
-    capped_glu_kernel<bf16_t><<<SM_CDIV(n, 256), 256, 0, stream>>>(
+    capped_glu_kernel<bf16_t, SILU><<<SM_CDIV(n, 256), 256, 0, stream>>>(
         reinterpret_cast<const bf16_t*>(gu.data_ptr()), n, ff, (float)limit,
         reinterpret_cast<bf16_t*>(out.data_ptr()));
   else {
     SM_CHECK_F32(gu);
-    capped_glu_kernel<float><<<SM_CDIV(n, 256), 256, 0, stream>>>(
+    capped_glu_kernel<float, SILU><<<SM_CDIV(n, 256), 256, 0, stream>>>(
         gu.data_ptr<float>(), n, ff, (float)limit, out.data_ptr<float>());
   }
   SM_CHECK_LAUNCH();
   return out;
 }
+
+torch::Tensor capped_glu(torch::Tensor gu, double limit) { return glu_impl<false>(gu, limit); }
+torch::Tensor silu_glu(torch::Tensor gu) { return glu_impl<true>(gu, 0.0); }

@@ -34,8 +34,9 @@ def _bf16(dtype) -> bool:
 def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0):
     """x / rms(x) * (offset + w) -> (fp32, out_dtype) rows."""
     if x.is_cuda:
-        return _ext("offset_rmsnorm").offset_rmsnorm(x.contiguous(), w, eps,
-                                                     _bf16(out_dtype), offset)
+        return _ext("offset_rmsnorm").offset_rmsnorm(
+            x if x.stride(-1) == 1 else x.contiguous(), w, eps,
+            _bf16(out_dtype), offset)
     return R.offset_rmsnorm(x, w, eps, out_dtype, offset)
 
 
