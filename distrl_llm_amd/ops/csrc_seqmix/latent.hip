@@ -83,8 +83,11 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
 template <typename T>
 SM_INLINE float lat_close(float M, float L, const float* sink, const T* gate, int64_t ldg,
                           int64_t t, int hd) {
-  if (sink != nullptr) L += expf(sink[hd] - M);
   float f = 1.0f / L;
+  if (sink != nullptr) {
+    const float M2 = fmaxf(M, sink[hd]), e = expf(M - M2);
+    f = e / (L * e + expf(sink[hd] - M2));
+  }
   if (gate != nullptr) f *= sm_sigmoid(to_f(gate[t * ldg + hd]));
   return f;
 }

@@ -211,3 +211,119 @@ def forward(cfg, w, tokens, layers_out=None):
             layers_out.append(x.clone())
     hid = unit_rms(x, eps) * w["final.norm"]
     return hid @ w["embed"].T * float(cfg["logit_scale"])
+
+
+# ------------------------------------------------ configurations and weights
+
+def latent_layer(heads=2, dim=4, rot_dim=4, vdim=5, kv_rank=6, q_rank=7, scale=0.4,
+                 base=100.0, rot_dims=None, scaling=None, mlp=8):
+    rot = {"base": base, "dims": rot_dim if rot_dims is None else rot_dims}
+    if scaling is not None:
+        rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return {"type": "latent_attention", "mlp": _mlp(mlp),
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim,
+                      "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale, "rot": rot}}
+
+
+def channel_layer(heads=2, kv_heads=2, dim=8, vdim=6, conv=3, mlp=None, ranks=(3, 5)):
+    return {"type": "channel_delta", "mlp": _mlp(mlp), "ranks": ranks,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                      "conv": conv}}
+
+
+def parallel_layer(heads=4, kv_heads=2, dim=6, vdim=5, scale=0.5, window=5, keep=2,
+                   r_heads=2, r_kv_heads=1, r_dim=8, r_vdim=6, conv=2, left_scale=0.8,
+                   right_scale=1.3, mlp=8):
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if window:
+        left["mask"] = {"size": window, "keep_first": keep}
+    return {"type": "parallel", "mlp": _mlp(mlp),
+            "mixer": {"left": left, "left_scale": left_scale, "right_scale": right_scale,
+                      "right": {"heads": r_heads, "kv_heads": r_kv_heads, "dim": r_dim,
+                                "vdim": r_vdim, "conv": conv}}}
+
+
+def _mlp(ff):
+    return None if ff is None else {"kind": "dense", "ff": ff}
+
+
+def make_cfg(layers, width=16, vocab=29, eps=1e-5, embed_scale=0.7, logit_scale=0.4):
+    """(config dict, {layer index: (decay rank, gate rank)})."""
+    ranks = {i: l["ranks"] for i, l in enumerate(layers) if "ranks" in l}
+    layers = [{k: v for k, v in l.items() if k != "ranks"} for l in layers]
+    return {"architecture": "Kakilorn", "embedding": {"scale": embed_scale},
+            "layers": layers, "logit_scale": logit_scale, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}, ranks
+
+
+def random_weights(cfg, ranks, seed=0):
+    """Random bf16-representable tensors under the design's names."""
+    g = torch.Generator().manual_seed(seed)
+    D = cfg["width"]
+    w = {}
+
+    def mat(name, rows, cols, s=None):
+        w[name] = torch.randn(rows, cols, generator=g) * (s if s is not None else cols ** -0.5)
+
+    def vec(name, n, mean=0.0, s=0.3):
+        w[name] = mean + s * torch.randn(n, generator=g)
+
+    def delta(x, mc, chan, rk=None):
+        H, G, dk, dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        for nm, rows in (("q", G * dk), ("k", G * dk), ("v", H * dv)):
+            mat(x + nm, rows, D, 1.5 * D ** -0.5)
+            mat(x + nm + ".conv", rows, mc["conv"], 0.6)
+        mat(x + "b", H, D)
+        vec(x + "A_log", H, -0.5, 0.5)
+        vec(x + "norm", dv, 1.0, 0.2)
+        if chan:
+            mat(x + "a1", rk[0], D)
+            mat(x + "a2", H * dk, rk[0])
+            vec(x + "dt_bias", H * dk, -1.0, 1.0)
+            mat(x + "g1", rk[1], D)
+            mat(x + "g2", H * dv, rk[1])
+        else:
+            mat(x + "a", H, D)
+            vec(x + "dt_bias", H, -1.0, 1.0)
+            mat(x + "g", H * dv, D)
+        mat(x + "o", D, H * dv)
+
+    mat("embed", cfg["vocab"], D, 1.0)
+    vec("final.norm", D, 1.0, 0.2)
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc = f"l{i}.", lc["mixer"]
+        x = p + "mix."
+        vec(p + "norm1", D, 1.0, 0.2)
+        if lc["type"] == "latent_attention":
+            H, dn, dr, dv = mc["heads"], mc["dim"], mc["rot_dim"], mc["vdim"]
+            r, rq = mc["kv_rank"], mc["q_rank"]
+            mat(x + "dq", rq, D)
+            vec(x + "dq.norm", rq, 1.0, 0.2)
+            mat(x + "uq", H * (dn + dr), rq, 2.0 * rq ** -0.5)
+            mat(x + "dkv", r + dr, D)
+            vec(x + "dkv.norm", r, 1.0, 0.2)
+            mat(x + "uk", H * dn, r, 2.0 * r ** -0.5)
+            mat(x + "uv", H * dv, r)
+            vec(x + "sink", H, 0.5, 1.0)
+            mat(x + "g", H, D)
+            mat(x + "o", D, H * dv)
+        elif lc["type"] == "channel_delta":
+            delta(x, mc, True, ranks[i])
+        else:
+            a = mc["left"]
+            H, G, dk, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            mat(x + "left.q", H * dk, D)
+            mat(x + "left.k", G * dk, D)
+            mat(x + "left.v", G * dv, D)
+            vec(x + "left.q.norm", dk, 1.0, 0.3)
+            vec(x + "left.k.norm", dk, 1.0, 0.3)
+            vec(x + "left.pb", H, -0.5, 0.7)
+            mat(x + "left.o", D, H * dv)
+            delta(x + "right.", mc["right"], False)
+        if lc.get("mlp") is not None:
+            ff = lc["mlp"]["ff"]
+            vec(p + "norm2", D, 1.0, 0.2)
+            mat(p + "mlp.gate", ff, D)
+            mat(p + "mlp.up", ff, D)
+            mat(p + "mlp.down", D, ff)
+    return {k: v.bfloat16().float() for k, v in w.items()}

@@ -1,0 +1,670 @@
+"""Kakilorn (post-norm layer-list model: latent attention with sink and gate,
+channel-decay delta rule, sigmoid attention beside the delta rule) against
+the plain oracle in kakilorn_oracle.py.
+
+Every test builds its own small configuration and random weights. The
+``dev`` fixture runs each case on the CPU path and, marked ``gpu``, on the
+HIP kernels (fp32 and bf16 models).
+"""
+
+import json
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import kakilorn_oracle as O
+from distrl_llm_amd.config import EngineConfig, SamplingParams
+from distrl_llm_amd.engine.hybrid_engine import HybridEngine
+from distrl_llm_amd.models.hybrid import (HybridLM, kakilorn_spec_from_config,
+                                          rotary_frequencies,
+                                          save_kakilorn_checkpoint)
+from distrl_llm_amd.ops import seqmix as SM
+
+CASES = [pytest.param(("cpu", torch.float32), id="cpu-f32"),
+         pytest.param(("cuda", torch.float32), id="gpu-f32", marks=pytest.mark.gpu),
+         pytest.param(("cuda", torch.bfloat16), id="gpu-bf16", marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=CASES)
+def dev(request):
+    return request.param
+
+
+def tol(dtype):
+    # bf16 is a coarse check on these tiny widths; the same kernels are held
+    # to 2e-4 in fp32 and the bf16-only tiled kernel has a test of its own
+    return 2e-4 if dtype == torch.float32 else 0.12
+
+
+def rel_err(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    d = got - want
+    return float(d.pow(2).mean().sqrt() / want.pow(2).mean().sqrt().clamp_min(1e-9))
+
+
+def mixed_cfg():
+    """Every mixer twice with sizes unequal wherever the design allows:
+    q/k heads shared by 1, 2 and 3 value heads, taps 1-4, rot.dims below
+    rot_dim, with and without frequency rescaling, windows with and without
+    kept tokens, one attention without a window, layers without feed-forward."""
+    return O.make_cfg([
+        O.channel_layer(heads=4, kv_heads=2, dim=8, vdim=6, conv=3, ranks=(3, 5), mlp=None),
+        O.latent_layer(heads=3, dim=4, rot_dim=6, vdim=5, kv_rank=7, q_rank=9, rot_dims=4,
+                       scaling=(4.0, 16, 2.0, 0.5), mlp=10),
+        O.parallel_layer(heads=4, kv_heads=2, dim=6, vdim=5, window=5, keep=2, r_heads=3,
+                         r_kv_heads=1, r_dim=40, r_vdim=5, conv=4, mlp=8),
+        O.latent_layer(heads=2, dim=6, rot_dim=4, vdim=3, kv_rank=5, q_rank=4, scaling=None,
+                       base=50.0, mlp=None),
+        O.channel_layer(heads=2, kv_heads=2, dim=5, vdim=9, conv=1, ranks=(2, 2), mlp=12),
+        O.parallel_layer(heads=3, kv_heads=3, dim=8, vdim=7, window=7, keep=0, r_heads=2,
+                         r_kv_heads=2, r_dim=8, r_vdim=6, conv=2, left_scale=1.0,
+                         right_scale=0.25, mlp=None),
+        O.parallel_layer(heads=2, kv_heads=1, dim=8, vdim=8, window=0, keep=0, r_heads=1,
+                         r_kv_heads=1, r_dim=6, r_vdim=4, conv=3, mlp=8),
+    ], width=16, vocab=37)
+
+
+def make_model(cfg, ranks, W, dev):
+    device, dtype = dev
+    shapes = {f"l{i}.mix.{n}": (r,) for i, rk in ranks.items()
+              for n, r in (("a1", rk[0]), ("g1", rk[1]))}
+    model = HybridLM(kakilorn_spec_from_config(cfg, shapes=shapes), dtype=dtype, device=device)
+    model.load_tensors(W)
+    return model
+
+
+def build(cfg_ranks, dev, seed=0, blocks=64, block_size=4, slots=4, W=None):
+    cfg, ranks = cfg_ranks
+    W = W if W is not None else O.random_weights(cfg, ranks, seed)
+    model = make_model(cfg, ranks, W, dev)
+    eng = HybridEngine(model, EngineConfig(max_seq_length=4096, kv_block_size=block_size,
+                                           num_kv_blocks=blocks, num_state_slots=slots,
+                                           max_num_seqs=slots), device=torch.device(dev[0]))
+    return W, eng
+
+
+def run_portions(eng, tokens, cuts, capture=None):
+    q = eng.open_sequence()
+    out, at = [], 0
+    for n in cuts:
+        out.append(eng.step([(q, tokens[at:at + n])], [list(range(n))], capture=capture))
+        at += n
+    assert at == len(tokens)
+    eng.close_sequence(q)
+    return torch.cat(out)
+
+
+def toks(n, vocab, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def ints(v, device):
+    return torch.tensor(v, dtype=torch.int32, device=device)
+
+
+# ------------------------------------------------------ mechanisms alone
+
+def test_post_norm_residual(dev):
+    device, dtype = dev
+    g = torch.Generator().manual_seed(0)
+    T, D, eps = 5, 24, 1e-4
+    x = torch.randn(T, D, generator=g)
+    y = torch.randn(T, D, generator=g).to(dtype).float()
+    y2 = torch.randn(T, D, generator=g).to(dtype).float()
+    w = 1.0 + 0.3 * torch.randn(D, generator=g)
+    for second, a, b in ((None, 1.0, 1.0), (y2, 0.7, 1.9)):
+        s = a * y.double() + (b * second.double() if second is not None else 0.0)
+        want = x.double() + O.unit_rms(s, eps) * w.double()
+        xd = x.clone().to(device)
+        h = SM.sandwich_residual_norm(
+            xd, y.to(dtype).to(device), None if second is None else second.to(dtype).to(device),
+            w.to(device), None, eps, dtype, 0.0, a, b, cast_next=True)
+        assert rel_err(xd, want) < 1e-6
+        assert h.dtype == dtype and rel_err(h.float(), want) < (1e-6 if dtype == torch.float32 else 5e-3)
+
+
+def test_plain_norm_and_silu_glu(dev):
+    device, dtype = dev
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(4, 40, generator=g).to(dtype)
+    w = torch.randn(24, generator=g)
+    h32, hb = SM.offset_rmsnorm(x.to(device)[:, 8:32], w.to(device), 1e-3, dtype, 0.0)
+    want = O.unit_rms(x[:, 8:32].double(), 1e-3) * w.double()
+    assert rel_err(h32, want) < 1e-6 and hb.dtype == dtype
+    gu = torch.randn(6, 2 * 9, generator=g).to(dtype)
+    want = O.silu(gu[:, :9].double()) * gu[:, 9:].double()
+    assert rel_err(SM.silu_glu(gu.to(device)).float(), want) < (1e-6 if dtype == torch.float32 else 5e-3)
+
+
+def test_rotary_table():
+    """Frequencies and the cos/sin factor against the oracle's table, with
+    and without rescaling, also where the blend region is a single pair."""
+    for dims, base, sc in ((8, 100.0, None), (16, 1e4, (8.0, 512, 16.0, 1.0)),
+                           (12, 500.0, (2.0, 64, 1.0, 1.0)), (4, 10.0, (3.0, 8, 4.0, 0.25))):
+        rot = {"dims": dims, "base": base}
+        if sc:
+            rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), sc))
+        f, mag = rotary_frequencies(dims, base, sc)
+        fo, mo = O.rotary_table(rot)
+        assert f == pytest.approx(fo, rel=1e-12) and mag == pytest.approx(mo, rel=1e-12)
+
+
+def test_latent_prepare_pairs(dev):
+    """Pair rotation with tabulated frequencies on rot.dims < rot_dim, latent
+    norm, page rows, strided inputs."""
+    device, dtype = dev
+    H, dn, rd, r, dims, eps = 2, 3, 6, 7, 4, 1e-4
+    rot = {"base": 50.0, "dims": dims, "scaling": {"factor": 4.0, "original": 16, "fast": 2.0,
+                                                    "slow": 0.5}}
+    T = 6
+    g = torch.Generator().manual_seed(2)
+    wide = torch.randn(T, 5 + H * (dn + rd) + r + rd + 3, generator=g).bfloat16().float()
+    nw = torch.randn(r, generator=g)
+    pos = torch.tensor([0, 1, 2, 40, 41, 1000], dtype=torch.int32)
+    rows = torch.tensor([5, 0, 3, 9, 8, 1], dtype=torch.int32)
+    cache = torch.zeros(12, r + rd, dtype=dtype, device=device)
+    f, mag = rotary_frequencies(dims, 50.0, (4.0, 16, 2.0, 0.5))
+    wd = wide.to(device, dtype)
+    q0 = 5
+    d0 = q0 + H * (dn + rd)
+    q_rot = SM.latent_prepare(wd[:, q0:d0], wd[:, d0:d0 + r + rd], H, dn, rd, r, nw.to(device),
+                              eps, pos.to(device), 50.0, dims, rows.to(device), cache,
+                              torch.tensor(f, dtype=torch.float32, device=device), mag, True)
+    for t in range(T):
+        d = wide[t, d0:d0 + r + rd].double()
+        c = O.unit_rms(d[:r], eps) * nw.double()
+        kr = O.rotate_interleaved(d[r:], int(pos[t]), rot)
+        assert rel_err(cache[int(rows[t])].float(), torch.cat([c, kr])) < tol(dtype)
+        qh = wide[t, q0:d0].double().view(H, dn + rd)[:, dn:]
+        assert rel_err(q_rot[t], O.rotate_interleaved(qh, int(pos[t]), rot)) < 1e-5
+
+
+def _attention_case(device, dtype, H, G, dk, dv, bs, lengths, news, seed=0):
+    """A paged cache filled with random normed keys and values for rows of
+    the given lengths, whose last ``news`` tokens are the step's queries."""
+    g = torch.Generator().manual_seed(seed)
+    W = G * (dk + dv)
+    nblk = sum((n + bs - 1) // bs for n in lengths)
+    perm = torch.randperm(nblk, generator=g).tolist()
+    cache = torch.zeros((nblk + 1) * bs, W, dtype=dtype, device=device)
+    tables, kv, qs, pos, seq, cu = [], [], [], [], [], [0]
+    for b, (n, m) in enumerate(zip(lengths, news)):
+        nb = (n + bs - 1) // bs
+        tables.append([perm.pop() for _ in range(nb)])
+        rows = torch.randn(n, W, generator=g).to(dtype)
+        kv.append(rows.float())
+        idx = torch.tensor([tables[-1][j // bs] * bs + j % bs for j in range(n)])
+        cache[idx.to(device)] = rows.to(device)
+        qs.append(torch.randn(m, H, dk, generator=g).to(dtype))
+        pos += list(range(n - m, n))
+        seq += [b] * m
+        cu.append(cu[-1] + m)
+    width = max(len(t) for t in tables)
+    tables = [t + [0] * (width - len(t)) for t in tables]
+    return cache, tables, kv, torch.cat(qs), pos, seq, cu
+
+
+def _sigmoid_direct(q, kv, pos, seq, H, G, dk, dv, scale, window, keep, slopes, pb):
+    out = torch.zeros(q.shape[0], H, dv, dtype=torch.float64)
+    for t in range(q.shape[0]):
+        rows, p = kv[seq[t]].double(), pos[t]
+        for a in range(H):
+            gi = a // (H // G)
+            for j in range(p + 1):
+                if window > 0 and not (p - j < window or j < keep):
+                    continue
+                s = float(q[t, a].double() @ rows[j, gi * dk:(gi + 1) * dk]) * scale
+                wgt = 1.0 / (1.0 + math.exp(-(s - slopes[a] * (p - j) + pb[a])))
+                out[t, a] += wgt * rows[j, G * dk + gi * dv:G * dk + (gi + 1) * dv]
+    return out.reshape(q.shape[0], H * dv)
+
+
+@pytest.mark.parametrize("H,G,dk,dv,window,keep", [(4, 2, 6, 5, 5, 2), (3, 3, 8, 7, 7, 0),
+                                                    (2, 1, 8, 8, 0, 0), (6, 2, 16, 24, 9, 12)])
+def test_sigmoid_attention_op(dev, H, G, dk, dv, window, keep):
+    """Prompt portions and single tokens in one step against a direct sum."""
+    device, dtype = dev
+    bs, lengths, news = 4, [23, 9, 14, 1], [11, 1, 14, 1]
+    cache, tables, kv, q, pos, seq, cu = _attention_case(device, dtype, H, G, dk, dv, bs,
+                                                         lengths, news)
+    slopes = [2.0 ** (-8.0 * (a + 1) / H) for a in range(H)]
+    pb = [0.3 - 0.4 * a for a in range(H)]
+    tiles, mt = SM.query_tiles(news, SM.WIDE_QUERY_TILE)
+    got = SM.sigmoid_attention(
+        q.to(device), cache, H, G, dk, dv, ints(tables, device), bs, ints(cu, device),
+        ints(seq, device), ints(pos, device), 0.37, window, keep,
+        torch.tensor(slopes, device=device), torch.tensor(pb, device=device), dtype,
+        tiles=ints(tiles, device), max_tile=mt)
+    want = _sigmoid_direct(q.float(), kv, pos, seq, H, G, dk, dv, 0.37, window, keep, slopes, pb)
+    assert rel_err(got.float(), want) < (1e-5 if dtype == torch.float32 else 6e-3)
+
+
+def test_sigmoid_attention_edges(dev):
+    """One key made to stand out (large q.k, a value of its own) among keys
+    whose weights are driven to zero: it must count just inside the window,
+    among the kept first tokens and at page borders, and must not count just
+    outside either, from a prompt portion and from a single decoded token."""
+    device, dtype = dev
+    H, G, dk, dv, bs, window, keep = 2, 1, 8, 8, 4, 12, 3
+    n = 40
+    slopes, pb = [0.0, 0.0], [-30.0, -30.0]
+    for m in (1, 9):                                   # decoded token / portion
+        p = n - 1                                      # the last query's position
+        for j_star, seen in ((p - window + 1, True), (p - window, False), (keep - 1, True),
+                             (keep, False), (p, True), (p - 4, True), (p - 3, True)):
+            g = torch.Generator().manual_seed(3)
+            kvr = 0.05 * torch.randn(n, dk + dv, generator=g)
+            kvr[j_star, :dk] = 4.0
+            kvr[j_star, dk:] = torch.arange(1, dv + 1).float()
+            kvr = kvr.to(dtype)
+            q = torch.full((m, H, dk), 4.0).to(dtype)  # q.k* * scale = 64: weight ~ 1
+            nb = (n + bs - 1) // bs
+            table = list(range(nb - 1, -1, -1))
+            cache = torch.zeros((nb + 1) * bs, dk + dv, dtype=dtype, device=device)
+            idx = torch.tensor([table[j // bs] * bs + j % bs for j in range(n)])
+            cache[idx.to(device)] = kvr.to(device)
+            pos = list(range(n - m, n))
+            tiles, mt = SM.query_tiles([m], SM.WIDE_QUERY_TILE)
+            got = SM.sigmoid_attention(
+                q.to(device), cache, H, G, dk, dv, ints([table], device), bs, ints([0, m], device),
+                ints([0] * m, device), ints(pos, device), 0.5, window, keep,
+                torch.tensor(slopes, device=device), torch.tensor(pb, device=device), dtype,
+                tiles=ints(tiles, device), max_tile=mt)
+            last = got[-1].float().cpu().view(H, dv)
+            if seen:
+                assert rel_err(last[0], torch.arange(1, dv + 1).double()) < 2e-2, (m, j_star)
+            else:
+                assert float(last.abs().max()) < 1e-3, (m, j_star)
+
+
+def test_latent_sink_gate_op(dev):
+    """Sink and gate of the latent attention against a direct softmax, with a
+    far key made to stand out among hundreds (its latent is the one that
+    must come back)."""
+    device, dtype = dev
+    H, r, rd, bs, n, m = 3, 8, 4, 4, 300, 5
+    g = torch.Generator().manual_seed(4)
+    rows = (0.3 * torch.randn(n, r + rd, generator=g))
+    j_star = 17
+    rows[j_star, :r] = 3.0
+    rows = rows.to(dtype)
+    nb = (n + bs - 1) // bs
+    table = torch.randperm(nb, generator=g).tolist()
+    cache = torch.zeros((nb + 1) * bs, r + rd, dtype=dtype, device=device)
+    idx = torch.tensor([table[j // bs] * bs + j % bs for j in range(n)])
+    cache[idx.to(device)] = rows.to(device)
+    q_lat = torch.randn(H, m, r, generator=g)
+    q_lat[0] = 3.0                                      # head 0 looks for the far key
+    q_lat = q_lat.to(dtype)
+    q_rot = torch.randn(m, H, rd, generator=g)
+    sink = torch.tensor([0.5, 3.0, -2.0])
+    gate = torch.randn(m, H + 2, generator=g).to(dtype)
+    pos = list(range(n - m, n))
+    tiles, mt = SM.query_tiles([m])
+    got = SM.latent_window_attention(
+        q_lat.to(device), q_rot.to(device), cache, r, ints([table], device), bs,
+        ints([0, m], device), ints([0] * m, device), ints(pos, device), 0, 0.4, dtype,
+        tiles=ints(tiles, device), max_tile=mt, sink=sink.to(device),
+        gate=gate.to(device)[:, 1:1 + H])
+    R = rows.double()
+    for a in range(H):
+        for t in range(m):
+            s = (R[:pos[t] + 1, :r] @ q_lat[a, t].double()
+                 + R[:pos[t] + 1, r:] @ q_rot[t, a].double()) * 0.4
+            e = torch.exp(s - s.max())
+            den = e.sum() + math.exp(float(sink[a]) - float(s.max()))
+            want = (e / den) @ R[:pos[t] + 1, :r] * torch.sigmoid(gate[t, 1 + a].double())
+            assert rel_err(got[a, t].float(), want) < (1e-5 if dtype == torch.float32 else 1.5e-2)
+            if a == 0:                                  # the far key dominates head 0
+                assert float((e / den)[j_star]) > 0.5
+
+
+@pytest.mark.parametrize("H,G,dk,dv,R", [(2, 2, 8, 6, 3), (3, 1, 40, 5, 2), (4, 2, 5, 70, 7),
+                                          (1, 1, 72, 9, 1)])
+def test_channel_delta_op(dev, H, G, dk, dv, R):
+    """Per-channel decays and the sigmoid gate against the oracle's walk, two
+    rows of unequal length in one step, the state carried into a second step."""
+    device, dtype = dev
+    g = torch.Generator().manual_seed(5)
+    lens = [9, 4]
+    T = sum(lens)
+    C = 2 * G * dk + H * dv
+    qkv = torch.randn(T, C, generator=g).to(dtype)
+    gate = torch.randn(T, H * dv, generator=g).to(dtype)
+    ab = torch.randn(T, H + R, generator=g)
+    up = torch.randn(H * dk, R, generator=g)
+    a_log, dtb = 0.3 * torch.randn(H, generator=g), torch.randn(H * dk, generator=g) - 1.0
+    nw = 1.0 + 0.2 * torch.randn(dv, generator=g)
+    state = torch.zeros(3, H * dk * dv, device=device)
+    state[1] = 7.0                                      # another sequence's slot stays as it is
+    outs = []
+    for lo, hi in ((0, 5), (5, 9)):                     # row 0 in two steps, row 1 in the first
+        sel = list(range(lo, hi)) + (list(range(9, 13)) if lo == 0 else [])
+        cu = [0, hi - lo] + ([hi - lo + 4] if lo == 0 else [])
+        slots = [2, 0] if lo == 0 else [2]
+        outs.append(SM.gated_delta_rule(
+            qkv[sel].to(device), gate[sel].to(device), ab[sel].to(device), a_log.to(device),
+            dtb.to(device), nw.to(device), 1e-5, state, ints(cu, device), ints(slots, device),
+            H, G, dk, dv, dtype, decay_up=up.to(device), gate_sigmoid=True).float().cpu())
+    got = torch.cat([outs[0][:5], outs[1], outs[0][5:]])
+    assert float((state[1] - 7.0).abs().max()) == 0.0
+    x = qkv.double()
+    for a, e in ((0, 9), (9, 13)):
+        q = x[a:e, :G * dk].view(-1, G, dk)
+        k = x[a:e, G * dk:2 * G * dk].view(-1, G, dk)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        q, k = q.repeat_interleave(H // G, 1), k.repeat_interleave(H // G, 1)
+        v = x[a:e, 2 * G * dk:].view(-1, H, dv)
+        step = torch.nn.functional.softplus(ab[a:e, H:].double() @ up.double().T + dtb.double())
+        decay = torch.exp(-torch.exp(a_log.double())[None, :, None] * step.view(-1, H, dk))
+        o = O.delta_walk(q, k, v, torch.sigmoid(ab[a:e, :H].double()), decay)
+        want = (O.unit_rms(o, 1e-5) * nw.double()
+                * torch.sigmoid(gate[a:e].double().view(-1, H, dv))).reshape(e - a, H * dv)
+        assert rel_err(got[a:e], want) < (2e-5 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("which", ["channel", "latent", "parallel"])
+def test_single_layer_models(dev, which):
+    """Each mixer alone in a one-layer model, with and without a feed-forward."""
+    layer = {"channel": O.channel_layer(heads=3, kv_heads=1, dim=8, vdim=6, conv=4, mlp=8),
+             "latent": O.latent_layer(scaling=(8.0, 32, 4.0, 1.0), mlp=None),
+             "parallel": O.parallel_layer(mlp=8)}[which]
+    cfg = O.make_cfg([layer], width=16, vocab=23)
+    W, eng = build(cfg, dev)
+    t = toks(19, 23)
+    cap, lay = [], []
+    got = run_portions(eng, t, [19], capture=cap)
+    want = O.forward(cfg[0], W, t, lay)
+    assert rel_err(cap[0], lay[0]) < tol(dev[1])
+    assert rel_err(got, want) < tol(dev[1])
+
+
+# ------------------------------------------------------------ whole models
+
+def test_whole_prompt_and_layers(dev):
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev)
+    t = toks(41, 37)
+    cap, lay = [], []
+    got = run_portions(eng, t, [41], capture=cap)
+    want = O.forward(cfg[0], W, t, lay)
+    for i, (a, b) in enumerate(zip(cap, lay)):
+        assert rel_err(a, b) < tol(dev[1]), f"layer {i}"
+    assert rel_err(got, want) < tol(dev[1])
+
+
+def test_first_tokens(dev):
+    """One- and two-token sequences, and the first tokens of a longer one."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev)
+    for n in (1, 2, 3):
+        t = toks(n, 37, seed=n)
+        assert rel_err(run_portions(eng, t, [n]), O.forward(cfg[0], W, t)) < tol(dev[1])
+
+
+@pytest.mark.parametrize("cuts", [[1] * 30, [2] * 15, [7, 2, 2, 1, 11, 3, 4], [16, 14], [29, 1],
+                                  [3, 27]])
+def test_portions(dev, cuts):
+    """Prefill against token-by-token decoding and portions of several sizes,
+    down to two tokens, cut inside pages and windows."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev)
+    t = toks(30, 37, seed=5)
+    want = O.forward(cfg[0], W, t)
+    assert rel_err(run_portions(eng, t, cuts), want) < tol(dev[1])
+
+
+def test_portions_do_not_change_fp32_results(dev):
+    device, dtype = dev
+    if dtype != torch.float32:
+        pytest.skip("fp32 invariance")
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev)
+    t = toks(33, 37, seed=6)
+    whole = run_portions(eng, t, [33])
+    for cuts in ([1] * 33, [2, 3, 5, 1, 9, 13], [17, 16]):
+        assert rel_err(run_portions(eng, t, cuts), whole) < 1e-5
+
+
+def test_mixed_batches_and_reuse(dev):
+    """Unequal requests in one step (portions beside single tokens, requests
+    sitting steps out), pages and slots given back and taken again; every
+    position against the oracle and against the request run alone."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev, blocks=40, slots=3)
+    V = 37
+    reqs = {k: toks(n, V, seed=10 + i) for i, (k, n) in
+            enumerate((("a", 26), ("b", 9), ("c", 17), ("d", 22), ("e", 5)))}
+    plan = [[("a", 7), ("b", 2)], [("a", 1), ("b", 3), ("c", 9)], [("a", 1), ("c", 2)],
+            [("a", 6), ("b", 4), ("c", 1)], [("c", 5), ("a", 1)], [("a", 10), ("d", 3)],
+            [("d", 1), ("e", 2)], [("d", 12), ("e", 1)], [("d", 6), ("e", 2)]]
+    live, at, got = {}, {k: 0 for k in reqs}, {k: [] for k in reqs}
+    for stepn in plan:
+        work, want = [], []
+        for k, n in stepn:
+            if k not in live:
+                live[k] = eng.open_sequence()
+            work.append((live[k], reqs[k][at[k]:at[k] + n]))
+            want.append(list(range(n)))
+        out = eng.step(work, want)
+        o = 0
+        for k, n in stepn:
+            got[k].append(out[o:o + n])
+            o += n
+            at[k] += n
+            if at[k] == len(reqs[k]):
+                eng.close_sequence(live.pop(k))
+    assert not live
+    _, solo = build(cfg, dev, W=W)
+    for k, t in reqs.items():
+        g = torch.cat(got[k])
+        assert rel_err(g, O.forward(cfg[0], W, t)) < tol(dev[1]), k
+        alone = run_portions(solo, t, [len(t)])
+        assert rel_err(g, alone) < (1e-5 if dev[1] == torch.float32 else 0.06), k
+
+
+def test_dirty_pages_and_slots(dev):
+    """A freed slot and freed pages hold another request's leftovers."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev, blocks=12, slots=1)
+    a, b = toks(40, 37, seed=20), toks(35, 37, seed=21)
+    run_portions(eng, a, [40])
+    for t in eng.slots._tensors():
+        t.add_(3.0)                                    # whatever a previous owner left
+    for r in eng.pool.rows.values():
+        r.add_(5.0)
+    assert rel_err(run_portions(eng, b, [20, 15]), O.forward(cfg[0], W, b)) < tol(dev[1])
+
+
+def test_long_decode_past_windows(dev):
+    """120 single-token steps: every window passes over decoded tokens, the
+    kept first tokens stay, the recurrent state is carried."""
+    cfg = O.make_cfg([O.parallel_layer(window=9, keep=3, mlp=8),
+                      O.latent_layer(mlp=None),
+                      O.channel_layer(mlp=8),
+                      O.parallel_layer(heads=2, kv_heads=2, window=16, keep=5, mlp=None)],
+                     width=16, vocab=31)
+    W, eng = build(cfg, dev, blocks=48)
+    t = toks(132, 31, seed=30)
+    got = run_portions(eng, t, [12] + [1] * 120)
+    want = O.forward(cfg[0], W, t)
+    assert rel_err(got, want) < tol(dev[1])
+    assert rel_err(got[-20:], want[-20:]) < tol(dev[1])
+
+
+def test_window_edges_in_model(dev):
+    """Moving the token just inside a window, or the last kept one, changes a
+    later position's logits; the token just outside both does not."""
+    device, dtype = dev
+    cfg = O.make_cfg([O.parallel_layer(window=6, keep=2, right_scale=0.0, left_scale=1.0,
+                                       conv=1, mlp=None)], width=16, vocab=31)
+    W, eng = build(cfg, dev)
+    base = toks(20, 31, seed=40)
+    ref = run_portions(eng, base, [10, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1])[-1]
+    for j, seen in ((19 - 5, True), (19 - 6, False), (1, True), (2, False)):
+        alt = list(base)
+        alt[j] = (alt[j] + 7) % 31
+        for cuts in ([20], [10] + [1] * 10):
+            out = run_portions(eng, alt, cuts)[-1]
+            moved = rel_err(out, ref)
+            assert (moved > 1e-3) == seen, (j, cuts, moved)
+            assert rel_err(out, O.forward(cfg[0], W, alt)[-1]) < tol(dtype)
+
+
+def test_other_sizes(dev):
+    """Values a model may happen to make equal or 1: one head, one q/k head,
+    one tap, rank 1, equal sizes everywhere, unit scales, no rescaling."""
+    cfg = O.make_cfg([
+        O.latent_layer(heads=1, dim=8, rot_dim=8, vdim=8, kv_rank=8, q_rank=8, scale=1.0,
+                       mlp=16),
+        O.channel_layer(heads=1, kv_heads=1, dim=8, vdim=8, conv=1, ranks=(1, 1), mlp=16),
+        O.parallel_layer(heads=1, kv_heads=1, dim=8, vdim=8, scale=1.0, window=1, keep=1,
+                         r_heads=1, r_kv_heads=1, r_dim=8, r_vdim=8, conv=1, left_scale=1.0,
+                         right_scale=1.0, mlp=16),
+    ], width=8, vocab=11, embed_scale=1.0, logit_scale=1.0)
+    W, eng = build(cfg, dev)
+    t = toks(17, 11, seed=50)
+    want = O.forward(cfg[0], W, t)
+    assert rel_err(run_portions(eng, t, [17]), want) < tol(dev[1])
+    assert rel_err(run_portions(eng, t, [5, 2, 1, 9]), want) < tol(dev[1])
+
+
+def test_greedy_generate(dev):
+    """Greedy decoding through generate() and its scheduler (small step
+    budget, two prompts): every generated token is the oracle's argmax for
+    its prefix wherever the oracle's margin is not a rounding matter."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev, blocks=64, slots=4)
+    eng.cfg.step_token_budget = 8
+    prompts = [toks(13, 37, seed=60), toks(6, 37, seed=61)]
+    sp = SamplingParams(max_tokens=10, temperature=0.0, n=1)
+    outs = eng.generate(prompts, sp)
+    margin = 1e-3 if dev[1] == torch.float32 else 0.3
+    for p, o in zip(prompts, outs):
+        gen = o[0]
+        assert len(gen) == 10
+        logits = O.forward(cfg[0], W, p + gen)
+        for i, tok in enumerate(gen):
+            row = logits[len(p) - 1 + i]
+            top2 = torch.topk(row, 2).values
+            if float(top2[0] - top2[1]) > margin:
+                assert int(row.argmax()) == tok, (i, tok)
+    assert eng.slots.num_free == 4 and eng.pool.allocator.num_free == 64
+
+
+@pytest.mark.gpu
+def test_captured_decode_matches_eager():
+    cfg = mixed_cfg()
+    dev = ("cuda", torch.bfloat16)
+    W, eng = build(cfg, dev)
+    _, eager = build(cfg, dev, W=W)
+    eager.cfg.enforce_eager = True
+    t = toks(30, 37, seed=70)
+    a = run_portions(eng, t, [10] + [1] * 20)
+    b = run_portions(eager, t, [10] + [1] * 20)
+    assert rel_err(a, b) < 1e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dk,dv,window,keep,lengths,news", [
+    (4, 1, 40, 56, 150, 12, [300, 70, 5], [300, 64, 5]),
+    (2, 2, 128, 128, 64, 0, [200, 130], [70, 129]),
+    (8, 2, 64, 32, 0, 0, [150], [150]),
+    (3, 1, 32, 200, 40, 70, [260, 90], [200, 17]),
+    (2, 1, 256, 64, 100, 3, [180], [66]),
+])
+def test_tiled_sigmoid_attention_kernel(H, G, dk, dv, window, keep, lengths, news):
+    """The bf16 MFMA kernel against the one-wave kernel run in fp32 on the
+    same (bf16-rounded) inputs: tiles that start inside a window, kept tokens
+    inside and before the first window, pages in random order."""
+    device, bs = "cuda", 16
+    cache, tables, kv, q, pos, seq, cu = _attention_case(device, torch.bfloat16, H, G, dk, dv, bs,
+                                                         lengths, news, seed=9)
+    slopes = torch.tensor([2.0 ** (-8.0 * (a + 1) / H) for a in range(H)], device=device)
+    pb = torch.linspace(-1.0, 0.5, H, device=device)
+    tiles, mt = SM.query_tiles(news, SM.WIDE_QUERY_TILE)
+    args = (H, G, dk, dv, ints(tables, device), bs, ints(cu, device), ints(seq, device),
+            ints(pos, device), dk ** -0.5, window, keep, slopes, pb)
+    got = SM.sigmoid_attention(q.to(device), cache, *args, torch.bfloat16,
+                               tiles=ints(tiles, device), max_tile=mt)
+    want = SM.sigmoid_attention(q.float().to(device), cache.float(), *args, torch.float32)
+    assert rel_err(got.float(), want) < 6e-3
+
+
+# ------------------------------------------- checkpoints, registry, replay
+
+def test_checkpoint_registry_and_replay(tmp_path):
+    """Save a checkpoint, load it through the registry (the ranks of the
+    low-rank inputs come from the tensor shapes) and replay a step trace
+    through bin/trace_run: portions, a request that sits a step out, a slot
+    and pages taken again."""
+    cfg = mixed_cfg()
+    W = O.random_weights(*cfg, seed=3)
+    model = make_model(cfg[0], cfg[1], W, ("cpu", torch.float32))
+    path = str(tmp_path / "ckpt")
+    save_kakilorn_checkpoint(model, path)
+    with open(os.path.join(path, "config.json")) as f:
+        saved = json.load(f)
+    assert saved["architecture"] == "Kakilorn" and len(saved["layers"]) == 7
+
+    from distrl_llm_amd.models.registry import load_model_and_engine
+    m2, eng = load_model_and_engine(path, EngineConfig(max_seq_length=256, kv_block_size=4,
+                                                       num_kv_blocks=32, num_state_slots=2,
+                                                       max_num_seqs=2),
+                                    dtype=torch.float32, device=torch.device("cpu"))
+    assert m2.spec.layers == model.spec.layers
+    back = m2.export_tensors()
+    for k, v in W.items():
+        assert torch.equal(back[k].float(), v), k
+
+    a, b, c = toks(15, 37, seed=80), toks(7, 37, seed=81), toks(9, 37, seed=82)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]},
+                                {"id": "b", "tokens": b[:2], "want": []}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[6:8], "want": [1]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[2:], "want": [4]},
+                                {"id": "a", "tokens": a[8:], "want": [6]}], "end": ["a", "b"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [8]}], "end": ["c"]},
+    ]
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, CUDA_VISIBLE_DEVICES="", HIP_VISIBLE_DEVICES="")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path,
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "64",
+                        "--slots", "2", "--block-size", "4"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                       capture_output=True, env=env, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    import numpy as np
+    la, lb, lc = (O.forward(cfg[0], W, t) for t in (a, b, c))
+    want = {0: la[[0, 5]], 1: la[[7]], 2: torch.stack([lb[6], la[14]]), 3: lc[[8]]}
+    for i, w in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, 37))
+        assert rel_err(got, w) < 2e-4, i
+
+
+def test_config_errors():
+    cfg, ranks = O.make_cfg([O.parallel_layer(heads=3, kv_heads=2)])
+    with pytest.raises(ValueError, match="multiple of kv_heads"):
+        kakilorn_spec_from_config(cfg)
+    cfg, ranks = O.make_cfg([O.channel_layer()])
+    with pytest.raises(ValueError, match="ranks"):
+        kakilorn_spec_from_config(cfg)
+    cfg, ranks = O.make_cfg([O.latent_layer(rot_dim=4, rot_dims=6)])
+    with pytest.raises(ValueError, match="rot.dims"):
+        kakilorn_spec_from_config(cfg)
+    cfg, ranks = O.make_cfg([O.latent_layer()])
+    cfg["layers"][0]["type"] = "something"
+    with pytest.raises(ValueError, match="unknown mixer"):
+        kakilorn_spec_from_config(cfg)
+    cfg, ranks = O.make_cfg([O.latent_layer()])
+    cfg["layers"][0]["mlp"]["kind"] = "moe"
+    with pytest.raises(ValueError, match="unknown mlp"):
+        kakilorn_spec_from_config(cfg)
