@@ -1,5 +1,5 @@
 """Prefill and decode throughput of the layer-list designs (Nibalix,
-Nedasun) beside one another and beside the dense transformer of equal size
+Nedasun, Kakilorn) beside one another and beside the dense transformer of equal size
 (``bench.py --hybrid-bench``).
 
 All models get random weights at layer sizes that resemble a real model
@@ -78,12 +78,54 @@ def nedasun_bench_config(s: dict) -> dict:
             "vocab": s["vocab"], "width": s["width"]}
 
 
+def kakilorn_bench_config(s: dict) -> dict:
+    """Same width, depth and head count as the other designs of the size,
+    head sizes of the Nedasun config (128/128, 4 query heads per kv head)
+    and the latent sizes of the Nibalix config. Layer pattern: channel-decay
+    delta rule, latent attention, latent attention, sigmoid attention beside
+    the per-head delta rule; dense feed-forwards as wide as the experts one
+    token uses elsewhere (none after the first layer of each group)."""
+    kvh = max(1, s["heads"] // 4)
+    dense = {"kind": "dense", "ff": s["top"] * s["ff"]}
+    delta = {"heads": s["heads"], "kv_heads": kvh, "dim": 128, "vdim": 128, "conv": 4}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 4 == 0:
+            mc = dict(delta, decay_rank=s["width"] // 16, gate_rank=s["width"] // 16)
+            layers.append({"type": "channel_delta", "mixer": mc, "mlp": None})
+        elif i % 4 == 3:
+            left = {"heads": s["heads"], "kv_heads": kvh, "dim": 128, "vdim": 128,
+                    "scale": 128 ** -0.5,
+                    "mask": {"size": s["window"], "keep_first": 16}}
+            mc = {"left": left, "right": dict(delta, heads=s["heads"] // 2,
+                                              kv_heads=max(1, kvh // 2)),
+                  "left_scale": 1.0, "right_scale": 1.0}
+            layers.append({"type": "parallel", "mixer": mc, "mlp": dense})
+        else:
+            mc = {"heads": s["heads"], "dim": s["dim"], "rot_dim": s["rot_dim"],
+                  "vdim": s["vdim"], "kv_rank": s["kv_rank"],
+                  "q_rank": s["kv_rank"] * 3 // 2,
+                  "scale": (s["dim"] + s["rot_dim"]) ** -0.5,
+                  "rot": {"base": 10000.0, "dims": s["rot_dim"],
+                          "scaling": {"factor": 4.0, "original": 4096,
+                                      "fast": 32.0, "slow": 1.0}}}
+            layers.append({"type": "latent_attention", "mixer": mc, "mlp": dense})
+    return {"architecture": "Kakilorn", "embedding": {"scale": 1.0},
+            "layers": layers, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+            "vocab": s["vocab"], "width": s["width"]}
+
+
 def _build_hybrid(s, device, max_len, batch, design="nibalix"):
     from .engine.hybrid_engine import HybridEngine
-    from .models.hybrid import (HybridLM, nedasun_spec_from_config,
+    from .models.hybrid import (HybridLM, kakilorn_spec_from_config,
+                                nedasun_spec_from_config,
                                 nibalix_spec_from_config)
-    spec = (nedasun_spec_from_config(nedasun_bench_config(s)) if design == "nedasun"
-            else nibalix_spec_from_config(nibalix_bench_config(s)))
+    if design == "kakilorn":
+        spec = kakilorn_spec_from_config(kakilorn_bench_config(s))
+    elif design == "nedasun":
+        spec = nedasun_spec_from_config(nedasun_bench_config(s))
+    else:
+        spec = nibalix_spec_from_config(nibalix_bench_config(s))
     model = HybridLM(spec, dtype=torch.bfloat16, device=device).random_init(1)
     cfg = EngineConfig(max_seq_length=max_len, kv_block_size=16,
                        num_kv_blocks=batch * ((max_len + 15) // 16) + 8,
@@ -130,7 +172,7 @@ def measure(engine, vocab, batch, prompt_len, new_tokens, device):
             "prefill_s": t_pre, "decode_ms_per_step": 1e3 * dec / (new_tokens - 1)}
 
 
-def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("nedasun", "nibalix", "dense")):
+def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("kakilorn", "nedasun", "nibalix", "dense")):
     out = []
     for name in sizes:
         s = SIZES[name]
