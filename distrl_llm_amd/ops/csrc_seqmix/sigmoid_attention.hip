@@ -3,8 +3,10 @@
 // over the keys, under a sliding window that also keeps the first tokens.
 //   qk_norm_kv_write   per token: RMS norm of every q and k head over the head
 //                      size (plain shared weights), page write of [k | v]
-//   sigmoid_attention  one wave per (token, head): fp32 models, any shape,
-//                      steps of few tokens
+//   sigmoid_attention_group  decode steps: one workgroup per (token, kv
+//                      head, share of the keys) serves every query head of the
+//                      kv head, so a K/V row is read once for all of them
+//   sigmoid_attention  one wave per (token, head): any shape, the fallback
 // (the tiled MFMA kernel for bf16 prompt portions is in
 // sigmoid_attention_mfma.hip)
 // A query at position p sees the keys [0, min(keep, lo)) and [lo, p] with
@@ -106,6 +108,195 @@ __global__ __launch_bounds__(64) void sigmoid_attention_kernel(
   }
 }
 
+// ---- decode steps. One workgroup (4 waves) per (token, kv head g, key
+// share z). The REP query heads of g sit in LDS as fp32; the visible keys (one
+// list: kept first tokens before the window, then the window) are cut into
+// blocks of 64, share z takes a contiguous run of blocks and its waves take
+// them in turn. Per block: lane = key, the K row is read once in 16-byte
+// pieces and dotted with all REP queries; the REP x 64 fp32 weights go through
+// a wave-private LDS tile; then lane = pair of value columns, and every V row
+// is read once (coalesced) for all REP heads. The waves' sums meet in LDS.
+// Sigmoid weights are final as they are, so shares just add: with ksplit > 1
+// the workgroup leaves an fp32 partial and sigmoid_attention_sum adds them in
+// a fixed order.
+#define SGG_CP 2     // value column pairs per lane: vdim <= 256
+template <typename T> struct sg_vec;
+template <> struct sg_vec<bf16_t> {
+  static constexpr int N = 8;
+  SM_INLINE static void load(const bf16_t* p, float* o) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const unsigned int w[4] = {raw.x, raw.y, raw.z, raw.w};
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __uint_as_float(w[i] << 16);
+      o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  SM_INLINE static float2 load2(const bf16_t* p) {
+    const unsigned int w = *reinterpret_cast<const unsigned int*>(p);
+    return make_float2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+  }
+};
+template <> struct sg_vec<float> {
+  static constexpr int N = 4;
+  SM_INLINE static void load(const float* p, float* o) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+  SM_INLINE static float2 load2(const float* p) { return *reinterpret_cast<const float2*>(p); }
+};
+
+template <typename T, int REP>
+__global__ __launch_bounds__(256) void sigmoid_attention_group_kernel(
+    const T* __restrict__ q,          // [Tn, H, dk]
+    const T* __restrict__ cache,      // [rows, G dk + G vd]
+    const int* __restrict__ block_tables, int max_nb, int block_size,
+    const int* __restrict__ tok_seq, const int* __restrict__ positions, int H, int G,
+    int dk, int vd, float scale, int window, int keep,
+    const float* __restrict__ slopes, const float* __restrict__ pos_bias,
+    int ksplit, float* __restrict__ part,   // [ksplit, Tn, H, vd] when ksplit > 1
+    T* __restrict__ out) {                  // [Tn, H vd]
+  extern __shared__ __attribute__((aligned(16))) float sgl[];
+  constexpr int VN = sg_vec<T>::N;
+  float* qs = sgl;                                   // [REP][dk]
+  float* pw_all = qs + REP * dk;                     // [4][REP][64]
+  int* krow_all = reinterpret_cast<int*>(pw_all + 4 * REP * 64);   // [4][64]
+  float* red = reinterpret_cast<float*>(krow_all + 4 * 64);        // [3][REP][vd]
+  const int t = blockIdx.x, g = blockIdx.y, z = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t W = (int64_t)G * (dk + vd);
+  const int h0 = g * REP;
+  for (int i = tid; i < REP * dk; i += 256)
+    qs[i] = to_f(q[((int64_t)t * H + h0 + i / dk) * dk + i % dk]);
+  const int b = tok_seq[t], p = positions[t];
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int nfirst = (window > 0) ? min(keep, lo) : 0;
+  const int n = nfirst + (p - lo + 1);
+  const int nblk = (n + 63) / 64;
+  const int kb_lo = (int)(((int64_t)nblk * z) / ksplit);
+  const int kb_hi = (int)(((int64_t)nblk * (z + 1)) / ksplit);
+  const int* bt = block_tables + (int64_t)b * max_nb;
+  float* pw = pw_all + wave * REP * 64;
+  int* krow = krow_all + wave * 64;
+  float slope[REP], bias[REP];
+  #pragma unroll
+  for (int hh = 0; hh < REP; ++hh) { slope[hh] = slopes[h0 + hh]; bias[hh] = pos_bias[h0 + hh]; }
+  float acc[REP][SGG_CP][2];
+  #pragma unroll
+  for (int hh = 0; hh < REP; ++hh)
+    #pragma unroll
+    for (int c = 0; c < SGG_CP; ++c) acc[hh][c][0] = acc[hh][c][1] = 0.f;
+  __syncthreads();
+  for (int kb = kb_lo + wave; kb < kb_hi; kb += 4) {
+    const int i = kb * 64 + lane;
+    float s[REP];
+    #pragma unroll
+    for (int hh = 0; hh < REP; ++hh) s[hh] = 0.f;
+    int row = 0, j = 0;
+    if (i < n) {
+      j = (i < nfirst) ? i : lo + (i - nfirst);
+      row = bt[j / block_size] * block_size + j % block_size;
+      const T* kp = cache + (int64_t)row * W + g * dk;
+      for (int k = 0; k < dk; k += VN) {
+        float kv[VN];
+        sg_vec<T>::load(kp + k, kv);
+        #pragma unroll
+        for (int hh = 0; hh < REP; ++hh)
+          #pragma unroll
+          for (int e = 0; e < VN; ++e) s[hh] = fmaf(qs[hh * dk + k + e], kv[e], s[hh]);
+      }
+    }
+    #pragma unroll
+    for (int hh = 0; hh < REP; ++hh)
+      pw[hh * 64 + lane] =
+          (i < n) ? sm_sigmoid(s[hh] * scale - slope[hh] * (float)(p - j) + bias[hh]) : 0.f;
+    krow[lane] = row;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);              // the wave's LDS writes have landed
+    const int nk = min(64, n - kb * 64);
+    for (int jj = 0; jj < nk; ++jj) {
+      const T* vp = cache + (int64_t)krow[jj] * W + G * dk + g * vd;
+      #pragma unroll
+      for (int c = 0; c < SGG_CP; ++c) {
+        const int d = 2 * lane + 128 * c;
+        if (d < vd) {
+          const float2 v = sg_vec<T>::load2(vp + d);
+          #pragma unroll
+          for (int hh = 0; hh < REP; ++hh) {
+            const float w = pw[hh * 64 + jj];
+            acc[hh][c][0] = fmaf(w, v.x, acc[hh][c][0]);
+            acc[hh][c][1] = fmaf(w, v.y, acc[hh][c][1]);
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();                 // pw and krow are rewritten next round
+  }
+  // waves 1..3 leave their sums in LDS, wave 0 adds them in order and writes
+  if (wave > 0) {
+    #pragma unroll
+    for (int hh = 0; hh < REP; ++hh)
+      #pragma unroll
+      for (int c = 0; c < SGG_CP; ++c) {
+        const int d = 2 * lane + 128 * c;
+        if (d < vd) {
+          red[((wave - 1) * REP + hh) * vd + d] = acc[hh][c][0];
+          red[((wave - 1) * REP + hh) * vd + d + 1] = acc[hh][c][1];
+        }
+      }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  #pragma unroll
+  for (int hh = 0; hh < REP; ++hh)
+    #pragma unroll
+    for (int c = 0; c < SGG_CP; ++c) {
+      const int d = 2 * lane + 128 * c;
+      if (d < vd) {
+        float a0 = acc[hh][c][0], a1 = acc[hh][c][1];
+        for (int w = 0; w < 3; ++w) {
+          a0 += red[(w * REP + hh) * vd + d];
+          a1 += red[(w * REP + hh) * vd + d + 1];
+        }
+        if (ksplit > 1) {
+          float* dst = part + (((int64_t)z * gridDim.x + t) * H + h0 + hh) * vd + d;
+          dst[0] = a0; dst[1] = a1;
+        } else {
+          T* dst = out + ((int64_t)t * H + h0 + hh) * vd + d;
+          dst[0] = from_f<T>(a0); dst[1] = from_f<T>(a1);
+        }
+      }
+    }
+}
+
+// out = sum over the key shares, in order.
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_attention_sum_kernel(
+    const float* __restrict__ part, int64_t n, int ksplit, T* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float a = 0.f;
+  for (int z = 0; z < ksplit; ++z) a += part[z * n + i];
+  out[i] = from_f<T>(a);
+}
+
+template <typename T>
+bool launch_group(int rep, dim3 grid, size_t lds, hipStream_t stream, const T* q, const T* cache,
+                  const int* bt, int max_nb, int bs, const int* tok_seq, const int* pos, int H,
+                  int G, int dk, int vd, float scale, int window, int keep, const float* slopes,
+                  const float* pb, int ksplit, float* part, T* out) {
+#define SGG_CASE(R)                                                                         \
+  if (rep == R) {                                                                           \
+    sigmoid_attention_group_kernel<T, R><<<grid, 256, lds, stream>>>(                       \
+        q, cache, bt, max_nb, bs, tok_seq, pos, H, G, dk, vd, scale, window, keep, slopes,  \
+        pb, ksplit, part, out);                                                             \
+    return true;                                                                            \
+  }
+  SGG_CASE(1) SGG_CASE(2) SGG_CASE(3) SGG_CASE(4) SGG_CASE(6) SGG_CASE(8)
+#undef SGG_CASE
+  return false;
+}
+
 }  // namespace
 
 torch::Tensor qk_norm_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
@@ -182,6 +373,59 @@ torch::Tensor sigmoid_attention(torch::Tensor q, torch::Tensor cache, int64_t he
   auto out = torch::empty({T, (int64_t)H * vd}, q.options());
   if (T == 0) return out;
   auto stream = at::cuda::getCurrentCUDAStream();
+  const bool is_bf16 = q.scalar_type() == at::kBFloat16;
+  const int rep = H / G, vn = is_bf16 ? 8 : 4;
+  const bool rep_ok = rep <= 4 || rep == 6 || rep == 8;
+  // steps of few tokens per row: the grouped kernel, when the head sizes
+  // allow 16-byte pieces of K and column pairs of V
+  if (rep_ok && dk % vn == 0 && vd % 2 == 0 && ((int64_t)G * (dk + vd)) % vn == 0 &&
+      vd <= 128 * SGG_CP && (max_tile_queries <= 4 || !is_bf16) &&
+      (size_t)(rep * dk + 4 * rep * 64 + 3 * rep * vd + 4 * 64) * 4 <= 64 * 1024) {
+    if (!is_bf16) SM_CHECK_F32(q);
+    const size_t ldsg = (size_t)(rep * dk + 4 * rep * 64 + 3 * rep * vd + 4 * 64) * 4;
+    // enough key shares to fill the chip, at least four 64-key blocks each
+    const int64_t longest = (window > 0) ? window + keep_first
+                                         : (int64_t)block_tables.size(1) * block_size;
+    int ksplit = (int)std::min<int64_t>(std::max<int64_t>(1, 512 / std::max<int64_t>(1, T * G)),
+                                        std::max<int64_t>(1, longest / 256));
+    ksplit = std::min(ksplit, 16);
+    torch::Tensor part;
+    float* pp = nullptr;
+    if (ksplit > 1) {
+      part = torch::empty({ksplit, T, (int64_t)H * vd}, q.options().dtype(at::kFloat));
+      pp = part.data_ptr<float>();
+    }
+    dim3 gg(T, G, ksplit);
+    bool ran;
+    if (is_bf16)
+      ran = launch_group<bf16_t>(rep, gg, ldsg, stream, reinterpret_cast<const bf16_t*>(q.data_ptr()),
+                                 reinterpret_cast<const bf16_t*>(cache.data_ptr()),
+                                 block_tables.data_ptr<int>(), (int)block_tables.size(1),
+                                 (int)block_size, tok_seq.data_ptr<int>(), positions.data_ptr<int>(),
+                                 H, G, dk, vd, (float)scale, (int)window, (int)keep_first,
+                                 slopes.data_ptr<float>(), pos_bias.data_ptr<float>(), ksplit, pp,
+                                 reinterpret_cast<bf16_t*>(out.data_ptr()));
+    else
+      ran = launch_group<float>(rep, gg, ldsg, stream, q.data_ptr<float>(), cache.data_ptr<float>(),
+                                block_tables.data_ptr<int>(), (int)block_tables.size(1),
+                                (int)block_size, tok_seq.data_ptr<int>(), positions.data_ptr<int>(),
+                                H, G, dk, vd, (float)scale, (int)window, (int)keep_first,
+                                slopes.data_ptr<float>(), pos_bias.data_ptr<float>(), ksplit, pp,
+                                out.data_ptr<float>());
+    TORCH_CHECK(ran, "sigmoid_attention: no grouped kernel for this head ratio");
+    SM_CHECK_LAUNCH();
+    if (ksplit > 1) {
+      const int64_t nel = T * (int64_t)H * vd;
+      if (is_bf16)
+        sigmoid_attention_sum_kernel<bf16_t><<<SM_CDIV(nel, 256), 256, 0, stream>>>(
+            pp, nel, ksplit, reinterpret_cast<bf16_t*>(out.data_ptr()));
+      else
+        sigmoid_attention_sum_kernel<float><<<SM_CDIV(nel, 256), 256, 0, stream>>>(
+            pp, nel, ksplit, out.data_ptr<float>());
+      SM_CHECK_LAUNCH();
+    }
+    return out;
+  }
   const size_t lds = (size_t)(dk + 64) * sizeof(float) + 64 * sizeof(int);
   dim3 grid(T, H);
   if (q.scalar_type() == at::kBFloat16)

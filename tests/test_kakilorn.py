@@ -599,6 +599,34 @@ def test_tiled_sigmoid_attention_kernel(H, G, dk, dv, window, keep, lengths, new
     assert rel_err(got.float(), want) < 6e-3
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,dk,dv,window,keep,lengths", [
+    (4, 1, 40, 56, 150, 12, [300, 70, 5]),          # four query heads per kv head
+    (6, 2, 32, 64, 0, 0, [700, 1]),                 # no window: the keys are split in shares
+    (8, 1, 16, 256, 64, 100, [260, 90, 33]),        # kept range longer than the window
+    (2, 2, 128, 130, 50, 4, [120]),                 # a value size that is not a multiple of 4
+])
+def test_grouped_sigmoid_attention_kernel(dtype, H, G, dk, dv, window, keep, lengths):
+    """Decode steps (one token per row): the kernel that serves all query
+    heads of a kv head at once, against a direct sum."""
+    device, bs = "cuda", 16
+    news = [1] * len(lengths)
+    cache, tables, kv, q, pos, seq, cu = _attention_case(device, dtype, H, G, dk, dv, bs,
+                                                         lengths, news, seed=11)
+    slopes = [2.0 ** (-8.0 * (a + 1) / H) for a in range(H)]
+    pb = [0.2 - 0.3 * a for a in range(H)]
+    tiles, mt = SM.query_tiles(news, SM.WIDE_QUERY_TILE)
+    got = SM.sigmoid_attention(
+        q.to(device), cache, H, G, dk, dv, ints(tables, device), bs, ints(cu, device),
+        ints(seq, device), ints(pos, device), dk ** -0.5, window, keep,
+        torch.tensor(slopes, device=device), torch.tensor(pb, device=device), dtype,
+        tiles=ints(tiles, device), max_tile=mt)
+    want = _sigmoid_direct(q.float(), kv, pos, seq, H, G, dk, dv, dk ** -0.5, window, keep,
+                           slopes, pb)
+    assert rel_err(got.float(), want) < (1e-5 if dtype == torch.float32 else 6e-3)
+
+
 # ------------------------------------------- checkpoints, registry, replay
 
 def test_checkpoint_registry_and_replay(tmp_path):
