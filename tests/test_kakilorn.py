@@ -560,6 +560,50 @@ def test_greedy_generate(dev):
     assert eng.slots.num_free == 4 and eng.pool.allocator.num_free == 64
 
 
+def test_fork_shares_pages_and_copies_state(dev):
+    """n-candidate fan-out: the fork shares the prompt's full pages and gets
+    copies of the partial page, the state matrices and the conv tails of
+    every unit, the pair's two sides included."""
+    cfg = mixed_cfg()
+    W, eng = build(cfg, dev, blocks=20, block_size=4)
+    t = toks(18, 37, seed=33)
+    q = eng.open_sequence()
+    eng.step([(q, t[:10])], [[]])
+    c = eng.fork_sequence(q)
+    tail2 = [(x + 3) % 37 for x in t[10:]]
+    out = eng.step([(q, t[10:]), (c, tail2)], [list(range(8)), list(range(8))])
+    assert rel_err(out[:8], O.forward(cfg[0], W, t)[10:]) < tol(dev[1])
+    assert rel_err(out[8:], O.forward(cfg[0], W, t[:10] + tail2)[10:]) < tol(dev[1])
+    eng.close_sequence(q)
+    eng.close_sequence(c)
+    assert eng.pool.allocator.num_free == 20
+
+
+def test_served_through_the_batcher():
+    """The server's app, batcher and sampler drive the design's engine like
+    any other: greedy completions repeat, sampled ones fan out."""
+    from fastapi.testclient import TestClient
+
+    from distrl_llm_amd.serve import create_app
+    from distrl_llm_amd.utils.tokenizer import ByteTokenizer
+    cfg = O.make_cfg([O.latent_layer(mlp=8), O.parallel_layer(mlp=None), O.channel_layer(mlp=8)],
+                     width=16, vocab=600)
+    _, eng = build(cfg, ("cpu", torch.float32), blocks=128, block_size=8, slots=8)
+    client = TestClient(create_app(eng, ByteTokenizer(vocab_size=600), "tiny-kakilorn"))
+    body = {"prompt": "2+2=", "max_tokens": 5, "temperature": 0.0}
+    a = client.post("/v1/completions", json=body).json()
+    b = client.post("/v1/completions", json=body).json()
+    assert a["choices"][0]["text"] == b["choices"][0]["text"]
+    assert a["usage"]["completion_tokens"] <= 5
+    r = client.post("/v1/completions", json={"prompt": ["abcd", "wxyz"], "max_tokens": 3,
+                                             "temperature": 1.0, "top_p": 0.9, "n": 2}).json()
+    assert len(r["choices"]) == 4
+    lp = client.post("/v1/completions", json={"prompt": "ab", "max_tokens": 3, "temperature": 0.0,
+                                              "logprobs": 1})
+    assert lp.status_code == 200
+    assert eng.pool.allocator.num_free == 128 and eng.slots.num_free == 8
+
+
 @pytest.mark.gpu
 def test_captured_decode_matches_eager():
     cfg = mixed_cfg()
