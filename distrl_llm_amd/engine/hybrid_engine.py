@@ -25,8 +25,9 @@ import torch.nn.functional as F
 
 from ..config import EngineConfig, SamplingParams
 from ..models.hybrid import (DeltaRuleSpec, GluSpec, HybridLM,
-                             LatentAttentionSpec, ParallelMixerSpec,
-                             SigmoidAttentionSpec, SinkAttentionSpec)
+                             LatentAttentionSpec, MlpSpec, ParallelMixerSpec,
+                             SigmoidAttentionSpec, SinkAttentionSpec,
+                             WindowAttentionSpec)
 from ..ops import functional as OF
 from ..ops import seqmix as SM
 from ..utils.trace import trace_range
@@ -407,6 +408,37 @@ class HybridEngine:
                                  max_tile=meta["max_wide_tile"])
         return F.linear(o, L.out_w)
 
+    def _mix_window_attention(self, i, m, L, hm, meta, proj=None, x32=None):
+        """Windowed softmax attention. Biases come with the projection GEMM;
+        q/k norm, rotation, the fold of the score-mixing matrix into the
+        queries and the page write are one kernel; distance bias, window,
+        softmax and output gate are the attention kernel's."""
+        if proj is None:
+            proj = F.linear(hm, L.in_w, L.in_b if m.qkv_bias else None)
+        cache = self.pool.unit_rows(i, m)
+        freqs, mag = None, 1.0
+        if m.rope_dims:
+            f, mag = m.rope_table()
+            freqs = self._const(("rope", i), lambda: torch.tensor(
+                f, dtype=torch.float64).to(torch.float32).to(self.device))
+        q = SM.qk_prepare_kv_write(
+            proj, m.heads, m.kv_heads, m.dim, m.vdim,
+            L.q_norm_w if m.qk_norm else None, L.k_norm_w if m.qk_norm else None,
+            self.spec.norm_eps, meta["positions"], freqs, mag,
+            L.talk if m.score_mix else None, meta["page_slot"], cache)
+        gate = None
+        if m.out_gate:
+            g0 = m.q_size + m.k_size + m.v_size
+            gate = proj[:, g0:g0 + m.heads]
+        o = SM.window_attention(
+            q, cache, m.heads, m.kv_heads, m.dim, m.vdim, m.score_mix,
+            meta["block_tables"], self.pool.block_size, meta["cu"],
+            meta["tok_seq"], meta["positions"], m.scale, m.window,
+            m.keep_first, L.dist_r1 if m.log_distance else None,
+            L.dist_r2 if m.log_distance else None, gate, self.dtype,
+            tiles=meta["wide_tiles"], max_tile=meta["max_wide_tile"])
+        return F.linear(o, L.out_w)
+
     def _mix_delta(self, i, m, L, hm, meta, proj=None, x32=None):
         if proj is None:
             proj = F.linear(hm, L.in_w)
@@ -444,6 +476,8 @@ class HybridEngine:
             return self._mix_sink_attention(key, m, W, hm, meta, shared, proj)
         if isinstance(m, SigmoidAttentionSpec):
             return self._mix_sigmoid_attention(key, m, W, hm, meta, proj, x32)
+        if isinstance(m, WindowAttentionSpec):
+            return self._mix_window_attention(key, m, W, hm, meta, proj, x32)
         if isinstance(m, DeltaRuleSpec):
             return self._mix_delta(key, m, W, hm, meta, proj, x32)
         return self._mix_mingru(key, m, W, hm, meta, proj, x32)
@@ -468,6 +502,14 @@ class HybridEngine:
             gu = F.linear(hb, L.gu_w)
             act = SM.silu_glu(gu) if f.act == "silu" else SM.capped_glu(gu, f.limit)
             return F.linear(act, L.down_w), None
+        if isinstance(f, MlpSpec):
+            return F.linear(SM.gelu_tanh(F.linear(hb, L.up_w)), L.down_w), None
+        if f.routing == "sigmoid":
+            idx, wts = SM.moe_route_sigmoid(hb, L.router_w, f.top)
+            if f.scale_input:
+                return SM.moe_experts_scaled_input(hb, idx, wts, L.exp_gu,
+                                                   L.exp_down), None
+            return SM.moe_experts(hb, idx, wts, L.exp_gu, L.exp_down), None
         if f.routing == "all":
             idx, wts = SM.moe_route_all(hb, L.router_w, L.correction, f.top,
                                         f.scale)
@@ -487,13 +529,15 @@ class HybridEngine:
             x = self._layers_sandwich(tokens, meta, capture)
         elif S.block == "post_norm":
             x = self._layers_post_norm(tokens, meta, capture)
+        elif S.block == "pre_norm":
+            x = self._layers_pre_norm(tokens, meta, capture)
         else:
             x = self._layers_parallel_gated(tokens, meta, capture)
         if want_rows.numel() == 0:
             return torch.empty(0, S.vocab_size, dtype=torch.float32,
                                device=x.device)
         _, hb = SM.offset_rmsnorm(x[want_rows], M.final_norm_w, S.norm_eps, dt,
-                                  S.norm_offset)
+                                  S.norm_offset, S.norm_groups)
         logits = F.linear(hb, M.head).float()
         return logits * S.logit_scale if S.logit_scale != 1.0 else logits
 
@@ -577,6 +621,31 @@ class HybridEngine:
                 f, f2 = self._ff(ls.mlp, L, hb)
                 hb = SM.sandwich_residual_norm(x, f, f2, L.ff_post_w, None, eps,
                                                dt, off, cast_next=True)
+            if capture is not None:
+                capture.append(x.clone())
+        return x
+
+    def _layers_pre_norm(self, tokens, meta, capture):
+        """x += mixer(norm(x)), then x += ff(norm(x)): each sublayer reads a
+        (grouped) RMS norm of the fp32 residual and its output is added as it
+        is. The residual sum and the norm the next sublayer reads are one
+        kernel."""
+        S, M, dt = self.spec, self.model, self.dtype
+        eps, off, ng = S.norm_eps, S.norm_offset, S.norm_groups
+        shared = {}
+        x = M.embed[tokens].float()
+        if S.embed_scale != 1.0:
+            x = x * S.embed_scale
+        _, hb = SM.offset_rmsnorm(x, M.layers[0].norm_w, eps, dt, off, ng)
+        last = S.num_layers - 1
+        for i, (ls, L) in enumerate(zip(S.layers, M.layers)):
+            y = self._mixer(i, ls, L, hb, meta, shared)[0]
+            nxt = M.layers[i + 1].norm_w if i < last else None
+            hb = SM.residual_add_norm(
+                x, y, L.ff_norm_w if ls.mlp is not None else nxt, eps, dt, off, ng)
+            if ls.mlp is not None:
+                f, _ = self._ff(ls.mlp, L, hb)
+                hb = SM.residual_add_norm(x, f, nxt, eps, dt, off, ng)
             if capture is not None:
                 capture.append(x.clone())
         return x

@@ -27,7 +27,8 @@ import torch
 
 from ..models.hybrid import (DeltaRuleSpec, HybridSpec, LatentAttentionSpec,
                              MinGRUSpec, SigmoidAttentionSpec,
-                             SinkAttentionSpec, mixer_units)
+                             SinkAttentionSpec, WindowAttentionSpec,
+                             mixer_units)
 from .kvcache import BlockAllocator
 
 
@@ -49,7 +50,8 @@ class LatentCachePool:
 
     @staticmethod
     def _owns_rows(m) -> bool:
-        return (isinstance(m, (SinkAttentionSpec, SigmoidAttentionSpec))
+        return (isinstance(m, (SinkAttentionSpec, SigmoidAttentionSpec,
+                               WindowAttentionSpec))
                 or (isinstance(m, LatentAttentionSpec) and m.kv_from is None))
 
     def layer_rows(self, spec: HybridSpec, layer: int) -> torch.Tensor:

@@ -54,6 +54,23 @@ parameter, so another design can reuse them in another order.
   head, a sliding window that also keeps the first tokens) beside the
   per-head gated delta rule, summed with fixed scales;
 * feed-forward: a dense SiLU-gated GLU.
+
+``Legilix`` is the fourth:
+
+* residual stream in fp32, pre-norm sublayers ``x += mixer(norm(x))`` then
+  ``x += ff(norm(x))``; the norm is an RMS norm taken separately over equal
+  consecutive groups of the width (plain weights); scaled embedding that
+  also serves as the output matrix;
+* mixers: two forms of grouped-query softmax attention with q/k/v biases
+  under a sliding window (:class:`WindowAttentionSpec`): one with RMS-normed
+  queries and keys, half-layout rotary on part of each head with rescaled
+  frequencies, the heads' *scores* mixed by a learned matrix before the
+  softmax and a window that keeps the first tokens; one without rotation,
+  with a logarithmic distance bias per head and a per-head sigmoid output
+  gate;
+* feed-forward: a plain two-matrix MLP with tanh-GELU, or a mixture of
+  SiLU-gated experts routed by sigmoid scores that are not renormalised and
+  scale the expert's *input*.
 """
 
 from __future__ import annotations
@@ -246,6 +263,60 @@ class SigmoidAttentionSpec:
 
 
 @dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Grouped-query softmax attention over paged [k | v] rows under a
+    sliding window that may keep the first ``keep_first`` tokens. Options,
+    each off by default: biases on q/k/v, RMS norm of every q and k head
+    (plain shared weights), half-layout rotary (entry i pairs with
+    i + dims/2) on the first ``rope_dims`` entries with optionally rescaled
+    frequencies, mixing of the heads' scores by a learned [H, H] matrix
+    before the softmax, a distance bias ``-r1_h ln(1 + r2_h (i - j))`` and a
+    per-head sigmoid gate read from the mixer input."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0         # 0 = unbounded causal
+    keep_first: int = 0
+    qkv_bias: bool = False
+    qk_norm: bool = False
+    rope_dims: int = 0
+    rope_base: float = 10000.0
+    rope_scaling: Optional[tuple] = None
+    score_mix: bool = False
+    log_distance: bool = False
+    out_gate: bool = False
+
+    kind = "window_attention"
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def k_size(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def v_size(self) -> int:
+        return self.kv_heads * self.vdim
+
+    @property
+    def in_size(self) -> int:          # [q | k | v | gate]
+        return (self.q_size + self.k_size + self.v_size
+                + (self.heads if self.out_gate else 0))
+
+    @property
+    def cache_width(self) -> int:      # one cache row = [k heads | v heads]
+        return self.k_size + self.v_size
+
+    def rope_table(self):
+        """(per-pair frequencies, factor on cos and sin) in double precision."""
+        return rotary_frequencies(self.rope_dims, self.rope_base, self.rope_scaling)
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec:
     """Two mixers that read the same input; the result is
     ``left_scale * left + right_scale * right``."""
@@ -308,13 +379,25 @@ class GluSpec:
 
 
 @dataclass(frozen=True)
+class MlpSpec:
+    """Plain two-matrix feed-forward ``down(act(up h))``; ``act``
+    "gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
+    ff: int
+    act: str = "gelu_tanh"
+
+
+@dataclass(frozen=True)
 class MoESpec:
     experts: int
     top: int
     ff: int
     # routing "chosen": softmax over the chosen logits; "all": softmax over
-    # every router output, choice by score + correction, weight = score * scale
+    # every router output, choice by score + correction, weight = score * scale;
+    # "sigmoid": score = sigmoid(logit), the largest are chosen, weight = score
     routing: str = "chosen"
+    # the weight multiplies the expert's input (expert(w h)) instead of its
+    # output
+    scale_input: bool = False
     identity: int = 0       # trailing router outputs that pass the input through
     scale: float = 1.0
     limit: float = 0.0      # 0: SiLU-gated experts; > 0: clamped GLU experts
@@ -324,7 +407,7 @@ class MoESpec:
 @dataclass(frozen=True)
 class LayerSpec:
     mixer: object
-    mlp: object         # MoESpec, GluSpec or None
+    mlp: object         # MoESpec, GluSpec, MlpSpec or None
 
 
 @dataclass(frozen=True)
@@ -338,13 +421,17 @@ class HybridSpec:
     layers: tuple = field(default_factory=tuple)
     # "parallel_gated": one norm feeds mixer and feed-forward, gated sum;
     # "sandwich": norm before and after each sublayer, one after the other;
-    # "post_norm": sublayers read the residual, only their output is normed
+    # "post_norm": sublayers read the residual, only their output is normed;
+    # "pre_norm": x += sublayer(norm(x)), nothing else
     block: str = "parallel_gated"
     design: str = "nibalix"
     norm_offset: float = 1.0    # norm weights act as (offset + w)
     embed_scale: float = 1.0
     logit_scale: float = 1.0
     tied_head: bool = False     # the embedding table is the output matrix
+    # norms are taken separately over this many equal consecutive parts of
+    # the width
+    norm_groups: int = 1
 
     @property
     def num_layers(self) -> int:
@@ -466,6 +553,16 @@ def _make_mixer_weights(mod, m, D, P, packed_input=True):
         mod.q_norm_w, mod.k_norm_w = P(m.dim, dt=f32), P(m.dim, dt=f32)
         mod.pos_bias = P(m.heads, dt=f32)
         mod.out_w = P(D, m.heads * m.vdim)
+    elif isinstance(m, WindowAttentionSpec):
+        if m.qkv_bias:                  # added by the projection GEMM
+            mod.in_b = P(m.in_size)
+        if m.qk_norm:
+            mod.q_norm_w, mod.k_norm_w = P(m.dim, dt=f32), P(m.dim, dt=f32)
+        if m.score_mix:
+            mod.talk = P(m.heads, m.heads, dt=f32)
+        if m.log_distance:
+            mod.dist_r1, mod.dist_r2 = P(m.heads, dt=f32), P(m.heads, dt=f32)
+        mod.out_w = P(D, m.heads * m.vdim)
     elif isinstance(m, DeltaRuleSpec):
         mod.conv_w = P(m.conv_channels, m.taps, dt=f32)
         mod.ab_w = P(m.ab_rows, D, dt=f32)      # [write strength; decay input]
@@ -507,6 +604,10 @@ class HybridLayer(nn.Module):
             self.post_w = P(D, dt=f32)
             if ls.mlp is not None:
                 self.ff_post_w = P(D, dt=f32)
+        elif spec.block == "pre_norm":
+            self.norm_w = P(D, dt=f32)
+            if ls.mlp is not None:
+                self.ff_norm_w = P(D, dt=f32)
         elif spec.block == "sandwich":
             self.norm_w = P(D, dt=f32)
             self.post_w = P(D, dt=f32)
@@ -530,9 +631,13 @@ class HybridLayer(nn.Module):
         f = ls.mlp
         if isinstance(f, GluSpec):
             self.gu_w, self.down_w = P(2 * f.ff, D), P(D, f.ff)
+        elif isinstance(f, MlpSpec):
+            self.up_w, self.down_w = P(f.ff, D), P(D, f.ff)
         elif f is not None:
             n = f.experts + f.identity
-            self.router_w, self.router_b = P(n, D, dt=f32), P(n, dt=f32)
+            self.router_w = P(n, D, dt=f32)
+            if f.routing != "sigmoid":
+                self.router_b = P(n, dt=f32)
             if f.routing == "all":
                 self.correction = P(n, dt=f32)
             self.exp_gu = P(f.experts, 2 * f.ff, D)
@@ -581,6 +686,8 @@ class HybridLM(nn.Module):
             return _nedasun_named_slices(self)
         if self.spec.design == "kakilorn":
             return _kakilorn_named_slices(self)
+        if self.spec.design == "legilix":
+            return _legilix_named_slices(self)
         out = {"embed": (self.embed, None), "embed.norm": (self.embed_norm_w, None),
                "final.norm": (self.final_norm_w, None), "head": (self.head, None)}
         D = self.spec.width
@@ -668,6 +775,8 @@ class HybridLM(nn.Module):
                 r = torch.eye(dst.shape[0], device=dev) + 0.2 * r
             elif last == "vmix":
                 r = 0.3 + 0.1 * r
+            elif last in ("r1", "r2"):
+                r = 0.5 + 0.1 * r.abs()
             elif last == "conv":
                 r *= 0.5
             elif dst.dim() >= 2 and "canon" not in name:
@@ -1099,3 +1208,154 @@ def save_kakilorn_checkpoint(model: HybridLM, path: str) -> None:
     save_file(model.export_tensors(), os.path.join(path, "model.safetensors"))
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(kakilorn_config_from_spec(model.spec), f, indent=1)
+
+
+# ---------------------------------------------------------------- Legilix
+
+def legilix_spec_from_config(cfg: dict, name: str = "legilix") -> HybridSpec:
+    """Map a Legilix ``config.json`` onto the generic layer specs."""
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc, typ = lc["mixer"], lc["type"]
+        heads, kvh = int(mc["heads"]), int(mc["kv_heads"])
+        if kvh < 1 or heads % kvh:
+            raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+        mask = mc.get("mask") or {}
+        common = dict(heads=heads, kv_heads=kvh, dim=int(mc["dim"]),
+                      vdim=int(mc["vdim"]), scale=float(mc["scale"]),
+                      window=int(mask.get("size") or 0), qkv_bias=True)
+        if typ == "attention":
+            rot = mc.get("rot") or {}
+            sc = rot.get("scaling")
+            mixer = WindowAttentionSpec(
+                **common, keep_first=int(mask.get("keep_first") or 0),
+                qk_norm=True, rope_dims=int(rot.get("dims") or 0),
+                rope_base=float(rot.get("base") or 10000.0),
+                rope_scaling=(None if not sc else
+                              (float(sc["factor"]), float(sc["original"]),
+                               float(sc["fast"]), float(sc["slow"]))),
+                score_mix=True)
+            if mixer.rope_dims > mixer.dim or mixer.rope_dims % 2:
+                raise ValueError(f"layer {i}: rot.dims must be even and <= dim")
+        elif typ == "attention_2":
+            mixer = WindowAttentionSpec(**common, log_distance=True, out_gate=True)
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {typ!r}")
+        fc, mlp = lc.get("mlp"), None
+        if fc is not None and fc.get("kind") == "dense":
+            mlp = MlpSpec(ff=int(fc["ff"]))
+        elif fc is not None and fc.get("kind") == "moe":
+            rc = fc["router"]
+            mlp = MoESpec(experts=int(rc["experts"]), top=int(rc["top"]),
+                          ff=int(fc["expert"]["ff"]), routing="sigmoid",
+                          scale_input=True)
+            if not 1 <= mlp.top <= mlp.experts:
+                raise ValueError(f"layer {i}: top must be in [1, experts]")
+        elif fc is not None:
+            raise ValueError(f"layer {i}: unknown mlp kind {fc.get('kind')!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    groups = int((cfg["norm"].get("groups")) or 1)
+    if groups < 1 or int(cfg["width"]) % groups:
+        raise ValueError("norm.groups must divide the width")
+    return HybridSpec(name=name, vocab_size=int(cfg["vocab"]),
+                      width=int(cfg["width"]),
+                      norm_eps=float(cfg["norm"]["eps"]), residual_mult=1.0,
+                      conv_taps=0, layers=tuple(layers), block="pre_norm",
+                      design="legilix", norm_offset=0.0,
+                      embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+                      logit_scale=float(cfg.get("logit_scale", 1.0)),
+                      tied_head=True, norm_groups=groups)
+
+
+def legilix_config_from_spec(spec: HybridSpec) -> dict:
+    """Inverse of :func:`legilix_spec_from_config` (checkpoint saving)."""
+    layers = []
+    for ls in spec.layers:
+        m = ls.mixer
+        mc = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+              "vdim": m.vdim, "scale": m.scale}
+        if m.score_mix:
+            typ = "attention"
+            if m.window:
+                mc["mask"] = {"size": m.window, "keep_first": m.keep_first}
+            rot = {"base": m.rope_base, "dims": m.rope_dims}
+            if m.rope_scaling:
+                rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"),
+                                          m.rope_scaling))
+            mc["rot"] = rot
+        else:
+            typ = "attention_2"
+            if m.window:
+                mc["mask"] = {"size": m.window}
+        f, fc = ls.mlp, None
+        if isinstance(f, MlpSpec):
+            fc = {"kind": "dense", "ff": f.ff}
+        elif f is not None:
+            fc = {"kind": "moe", "expert": {"ff": f.ff},
+                  "router": {"experts": f.experts, "top": f.top}}
+        layers.append({"type": typ, "mixer": mc, "mlp": fc})
+    return {"architecture": "Legilix", "embedding": {"scale": spec.embed_scale},
+            "layers": layers, "logit_scale": spec.logit_scale,
+            "norm": {"eps": spec.norm_eps, "groups": spec.norm_groups},
+            "vocab": spec.vocab_size, "width": spec.width}
+
+
+def _legilix_named_slices(model: "HybridLM") -> Dict[str, tuple]:
+    out = {"embed": (model.embed, None), "final.norm": (model.final_norm_w, None)}
+    for i, (ls, L) in enumerate(zip(model.spec.layers, model.layers)):
+        p, m = f"l{i}.", ls.mixer
+        x = p + "mix."
+        out[p + "norm1"] = (L.norm_w, None)
+        r0 = 0
+        for nm, rows in (("q", m.q_size), ("k", m.k_size), ("v", m.v_size)):
+            out[x + nm] = (L.in_w, (r0, rows))
+            out[x + nm + ".b"] = (L.in_b, (r0, rows))
+            r0 += rows
+        if m.out_gate:                  # its rows of the packed bias stay zero
+            out[x + "g"] = (L.in_w, (r0, m.heads))
+        if m.qk_norm:
+            out[x + "q.norm"], out[x + "k.norm"] = (L.q_norm_w, None), (L.k_norm_w, None)
+        if m.score_mix:
+            out[x + "talk"] = (L.talk, None)
+        if m.log_distance:
+            out[x + "r1"], out[x + "r2"] = (L.dist_r1, None), (L.dist_r2, None)
+        out[x + "o"] = (L.out_w, None)
+        f = ls.mlp
+        if f is None:
+            continue
+        out[p + "norm2"] = (L.ff_norm_w, None)
+        x = p + "mlp."
+        if isinstance(f, MlpSpec):
+            out[x + "up"], out[x + "down"] = (L.up_w, None), (L.down_w, None)
+            continue
+        out[x + "router"] = (L.router_w, None)
+        for e in range(f.experts):
+            out[f"{x}e{e}.gate"] = (L.exp_gu[e], (0, f.ff))
+            out[f"{x}e{e}.up"] = (L.exp_gu[e], (f.ff, f.ff))
+            out[f"{x}e{e}.down"] = (L.exp_down[e], None)
+    return out
+
+
+def load_legilix_checkpoint(path: str, dtype=torch.bfloat16, device=None) -> HybridLM:
+    from safetensors.torch import load_file
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    name = os.path.basename(os.path.normpath(path)) or "legilix"
+    model = HybridLM(legilix_spec_from_config(cfg, name), dtype=dtype, device=device)
+    tensors = load_file(os.path.join(path, "model.safetensors"))
+    known = model._named_slices()
+    extra = sorted(k for k in tensors if k not in known)
+    if extra:
+        import sys
+        sys.stderr.write(f"[legilix] ignoring {len(extra)} tensors the design "
+                         f"does not name: {extra[:4]}\n")
+    model.load_tensors({k: v for k, v in tensors.items() if k in known})
+    return model
+
+
+def save_legilix_checkpoint(model: HybridLM, path: str) -> None:
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    save_file(model.export_tensors(), os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(legilix_config_from_spec(model.spec), f, indent=1)

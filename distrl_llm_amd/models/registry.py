@@ -69,11 +69,12 @@ def load_model_and_engine(path_or_name: str, engine_cfg, dtype=None,
 
 
 def _register_builtin():
-    from .hybrid import (load_kakilorn_checkpoint, load_nedasun_checkpoint,
-                         load_nibalix_checkpoint)
+    from .hybrid import (load_kakilorn_checkpoint, load_legilix_checkpoint,
+                         load_nedasun_checkpoint, load_nibalix_checkpoint)
     register_hybrid_design("Nibalix", load_nibalix_checkpoint)
     register_hybrid_design("Nedasun", load_nedasun_checkpoint)
     register_hybrid_design("Kakilorn", load_kakilorn_checkpoint)
+    register_hybrid_design("Legilix", load_legilix_checkpoint)
 
 
 _register_builtin()

@@ -31,13 +31,14 @@ def _bf16(dtype) -> bool:
     return dtype == torch.bfloat16
 
 
-def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0):
-    """x / rms(x) * (offset + w) -> (fp32, out_dtype) rows."""
+def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0, groups=1):
+    """x / rms(x) * (offset + w) -> (fp32, out_dtype) rows; ``groups`` > 1:
+    the root mean square of each of that many equal parts of the row."""
     if x.is_cuda:
         return _ext("offset_rmsnorm").offset_rmsnorm(
             x if x.stride(-1) == 1 else x.contiguous(), w, eps,
-            _bf16(out_dtype), offset)
-    return R.offset_rmsnorm(x, w, eps, out_dtype, offset)
+            _bf16(out_dtype), offset, groups)
+    return R.offset_rmsnorm(x, w, eps, out_dtype, offset, groups)
 
 
 def causal_tap_conv(h, w, tails, cu, tok_seq, slots, out_dtype):
@@ -165,22 +166,30 @@ def gated_residual_norm(x, mix, ff, gates, gate_b, mult, next_w, eps,
 
 def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
                            offset=1.0, y_scale=1.0, y2_scale=1.0,
-                           cast_next=False):
+                           cast_next=False, groups=1):
     """Fused sublayer tail: x += rms_unit(y_scale y [+ y2_scale y2]) *
-    (offset + post_w) on the fp32 residual (in place), then, with
-    ``next_w``, the next offset RMS norm of the new residual in
+    (offset + post_w) on the fp32 residual (in place; ``post_w`` None: the
+    sum is added without a closing norm), then, with ``next_w``, the next
+    offset RMS norm of the new residual (over ``groups`` equal parts) in
     ``out_dtype``; with ``cast_next`` instead the new residual itself in
     ``out_dtype`` (x when that is fp32); None without either."""
     if x.is_cuda:
         h = _ext("sandwich_residual_norm").sandwich_residual_norm(
             x, y.contiguous(), None if y2 is None else y2.contiguous(), post_w,
             next_w, eps, _bf16(out_dtype), offset, y_scale, y2_scale,
-            cast_next and next_w is None and _bf16(out_dtype))
+            cast_next and next_w is None and _bf16(out_dtype), groups)
         if h is None and cast_next and next_w is None:
             return x
         return h
     return R.sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
-                                    offset, y_scale, y2_scale, cast_next)
+                                    offset, y_scale, y2_scale, cast_next, groups)
+
+
+def residual_add_norm(x, y, next_w, eps, out_dtype, offset=1.0, groups=1):
+    """Pre-norm sublayer tail: x += y on the fp32 residual (in place), then,
+    with ``next_w``, the next norm of the new residual in ``out_dtype``."""
+    return sandwich_residual_norm(x, y, None, None, next_w, eps, out_dtype,
+                                  offset, groups=groups)
 
 
 def rope_kv_write(proj, heads, kv_heads, dim, vdim, positions, rope_base,
@@ -290,3 +299,59 @@ def moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit):
         return _ext("moe_experts_glu").moe_experts_glu(h, idx, wts, exp_gu,
                                                        exp_down, limit)
     return R.moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit)
+
+
+# ------------------------------------------- windowed softmax attention, MLP
+
+def qk_prepare_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w,
+                        eps, positions, freqs, mag, mix, page_slot, cache):
+    """``proj`` rows [q | k | v | ...] may be a column slice of a wider
+    matrix. ``q_norm_w``/``k_norm_w`` None: no q/k norm; ``freqs`` None: no
+    rotation; ``mix`` (fp32 [H, H]): the returned queries are folded with
+    the score-mixing matrix and span every kv head's key columns."""
+    if proj.is_cuda:
+        return _ext("qk_prepare_kv_write").qk_prepare_kv_write(
+            proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w, eps,
+            positions, freqs, mag, mix, page_slot, cache)
+    return R.qk_prepare_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w,
+                                 k_norm_w, eps, positions, freqs, mag, mix,
+                                 page_slot, cache)
+
+
+def window_attention(q, cache, heads, kv_heads, dim, vdim, whole_key,
+                     block_tables, block_size, cu, tok_seq, positions, scale,
+                     window, keep_first, r1, r2, gate, out_dtype, tiles=None,
+                     max_tile=0):
+    """``tiles`` (from :func:`query_tiles` with ``WIDE_QUERY_TILE``) selects
+    the tiled MFMA kernel for bf16 prompt portions; steps of few tokens per
+    row run one workgroup per (token, kv head, share of the keys), fp32
+    models and odd sizes one wave per (token, head). ``gate`` may be a
+    column slice of a wider matrix."""
+    if q.is_cuda:
+        return _ext("window_attention").window_attention(
+            q, cache, heads, kv_heads, dim, vdim, whole_key, block_tables,
+            block_size, tok_seq, positions, scale, window, keep_first, r1, r2,
+            gate, tiles, max_tile)
+    return R.window_attention(q, cache, heads, kv_heads, dim, vdim, whole_key,
+                              block_tables, block_size, cu, positions, scale,
+                              window, keep_first, r1, r2, gate, out_dtype)
+
+
+def gelu_tanh(x):
+    if x.is_cuda:
+        return _ext("gelu_tanh").gelu_tanh(x)
+    return R.gelu_tanh(x)
+
+
+def moe_route_sigmoid(h, router_w, top):
+    if h.is_cuda:
+        return _ext("moe_route_sigmoid").moe_route_sigmoid(h, router_w, top)
+    return R.moe_route_sigmoid(h, router_w, top)
+
+
+def moe_experts_scaled_input(h, idx, wts, exp_gu, exp_down):
+    """SiLU-gated experts whose routing weight multiplies their input."""
+    if h.is_cuda:
+        return _ext("moe_experts_scaled_input").moe_experts_scaled_input(
+            h, idx, wts, exp_gu, exp_down)
+    return R.moe_experts_scaled_input(h, idx, wts, exp_gu, exp_down)

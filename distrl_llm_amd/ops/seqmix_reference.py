@@ -18,10 +18,14 @@ import torch
 import torch.nn.functional as F
 
 
-def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0):
-    """x / sqrt(mean(x^2) + eps) * (offset + w) in fp32 -> (fp32, out_dtype)."""
+def offset_rmsnorm(x, w, eps, out_dtype, offset=1.0, groups=1):
+    """x / sqrt(mean(x^2) + eps) * (offset + w) in fp32 -> (fp32, out_dtype);
+    with ``groups`` > 1 the mean is taken separately over that many equal
+    consecutive parts of the row."""
     x = x.float()
-    h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
+    xg = x.view(x.shape[0], groups, -1)
+    h = (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).view_as(x)
+    h = h * (offset + w.float())
     return h, h.to(out_dtype)
 
 
@@ -221,18 +225,22 @@ def gated_residual_add(x, mix, ff, gates, gate_b, mult):
 
 def sandwich_residual_norm(x, y, y2, post_w, next_w, eps, out_dtype,
                            offset=1.0, y_scale=1.0, y2_scale=1.0,
-                           cast_next=False):
+                           cast_next=False, groups=1):
     """x += rms_unit(y_scale y [+ y2_scale y2]) * (offset + post_w) on the
-    fp32 residual, in place; with ``next_w`` also returns the next offset RMS
-    norm of the new residual in ``out_dtype``; with ``cast_next`` the new
+    fp32 residual, in place (``post_w`` None: the sum is added as it is);
+    with ``next_w`` also returns the next offset RMS norm of the new residual
+    (over ``groups`` parts) in ``out_dtype``; with ``cast_next`` the new
     residual itself in ``out_dtype``; else None."""
     s = y.float() * y_scale
     if y2 is not None:
         s = s + y2.float() * y2_scale
-    x.add_(s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps)
-           * (offset + post_w.float()))
+    if post_w is None:                  # no closing norm: the plain sum
+        x.add_(s)
+    else:
+        x.add_(s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + eps)
+               * (offset + post_w.float()))
     if next_w is not None:
-        return offset_rmsnorm(x, next_w, eps, out_dtype, offset)[1]
+        return offset_rmsnorm(x, next_w, eps, out_dtype, offset, groups)[1]
     return x.to(out_dtype) if cast_next else None
 
 
@@ -482,3 +490,116 @@ def moe_experts_glu(h, idx, wts, exp_gu, exp_down, limit):
         out[rows] += (wts[rows] * hit[rows]).sum(-1, keepdim=True) * y
     ident = (wts * (idx >= E)).sum(-1, keepdim=True)
     return out + ident * h.float()
+
+
+# ------------------------------------------- windowed softmax attention, MLP
+
+def qk_prepare_kv_write(proj, heads, kv_heads, dim, vdim, q_norm_w, k_norm_w,
+                        eps, positions, freqs, mag, mix, page_slot, cache):
+    """From packed [q | k | v | ...] projection rows: optional RMS norm of
+    every q and k head (plain shared weights), optional half-layout rotation
+    of their first 2 len(freqs) entries by position * freqs with cos and sin
+    scaled by ``mag``, page write of [k | v]. Returns the queries in the
+    projection's dtype: [T, heads, dim], or with ``mix`` (fp32 [H, H])
+    [T, heads, kv_heads * dim], where row h holds, in the columns of kv head
+    c, sum over the heads g of c of mix[h, g] q_g: its product with a whole
+    key row is the score of head h mixed over all heads."""
+    T = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q = proj[:, :nq].float().view(T, heads, dim)
+    k = proj[:, nq:nq + nk].float().view(T, kv_heads, dim)
+    if q_norm_w is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    if freqs is not None and freqs.numel():
+        q = _rotate_table(q, positions, freqs, mag, False)
+        k = _rotate_table(k, positions, freqs, mag, False)
+    v = proj[:, nq + nk:nq + nk + kv_heads * vdim].float()
+    cache[page_slot.long()] = torch.cat([k.reshape(T, nk), v], -1).to(cache.dtype)
+    if mix is not None:
+        rep = heads // kv_heads
+        m = mix.float().view(heads, kv_heads, rep)
+        q = torch.einsum("hcr,tcrd->thcd", m, q.view(T, kv_heads, rep, dim))
+        q = q.reshape(T, heads, nk)
+    return q.to(proj.dtype)
+
+
+def window_attention(q, cache, heads, kv_heads, dim, vdim, whole_key,
+                     block_tables, block_size, cu, positions, scale, window,
+                     keep_first, r1, r2, gate, out_dtype):
+    """Grouped-query softmax attention over paged [k | v] rows.
+
+    Query i sees the keys j <= i with i - j < window or j < keep_first
+    (window 0: all j <= i). score = q . k * scale, where head h meets the
+    keys of its own kv head, or with ``whole_key`` (q rows of kv_heads * dim
+    entries) the whole key row; ``r1``/``r2`` (fp32 [H]) take
+    r1 ln(1 + r2 (i - j)) off the score; ``gate`` ([T, H] pre-activations)
+    scales head h's result by its sigmoid. -> [T, H * vdim]."""
+    T = q.shape[0]
+    rep = heads // kv_heads
+    nk = kv_heads * dim
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32, device=q.device)
+    cu_l, pos_l = cu.tolist(), positions.tolist()
+    for b in range(len(cu_l) - 1):
+        a, e = cu_l[b], cu_l[b + 1]
+        if e == a:
+            continue
+        j = torch.arange(0, pos_l[e - 1] + 1, device=cache.device)
+        rows = block_tables[b].long()[j // block_size] * block_size + j % block_size
+        kv = cache[rows].float()
+        v = kv[:, nk:].view(-1, kv_heads, vdim).repeat_interleave(rep, 1)
+        if whole_key:
+            s = torch.einsum("thd,jd->htj", q[a:e].float(), kv[:, :nk]) * scale
+        else:
+            k = kv[:, :nk].view(-1, kv_heads, dim).repeat_interleave(rep, 1)
+            s = torch.einsum("thd,jhd->htj", q[a:e].float(), k) * scale
+        p = positions[a:e].long()[:, None]
+        if r1 is not None:
+            dist = (p - j[None, :]).clamp(min=0).float()
+            s = s - r1.float()[:, None, None] * torch.log1p(
+                r2.float()[:, None, None] * dist[None])
+        ok = j[None, :] <= p
+        if window > 0:
+            ok = ok & ((p - j[None, :] < window) | (j[None, :] < keep_first))
+        s = s.masked_fill(~ok[None], float("-inf"))
+        out[a:e] = torch.einsum("htj,jhd->thd", torch.softmax(s, -1), v)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[:, :, None]
+    return out.reshape(T, heads * vdim).to(out_dtype)
+
+
+def gelu_tanh(x):
+    """0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) in x's dtype."""
+    z = x.float()
+    return (0.5 * z * (1.0 + torch.tanh(0.7978845608028654
+                                        * (z + 0.044715 * z * z * z)))).to(x.dtype)
+
+
+def moe_route_sigmoid(h, router_w, top):
+    """fp32 router: scores = sigmoid(W h); the ``top`` largest (ties: lowest
+    index first); weights = the chosen scores, not renormalised."""
+    s = torch.sigmoid(F.linear(h.float(), router_w.float()))
+    _, idx = torch.sort(s, dim=-1, descending=True, stable=True)
+    idx = idx[:, :top]
+    return idx.to(torch.int32), torch.gather(s, 1, idx)
+
+
+def moe_experts_scaled_input(h, idx, wts, exp_gu, exp_down):
+    """sum_k down_e(silu(gate_e (w h)) * up_e (w h)), e = idx[t, k],
+    w = wts[t, k]: the weight multiplies the expert's input. The products
+    gate_e h and up_e h are scaled by w in fp32 before the activation.
+    Returns fp32 [T, D]."""
+    T, D = h.shape
+    E, ff2, _ = exp_gu.shape
+    ff = ff2 // 2
+    out = torch.zeros(T, D, dtype=torch.float32, device=h.device)
+    for k in range(idx.shape[1]):
+        for e in range(E):
+            rows = (idx[:, k] == e).nonzero().flatten()
+            if rows.numel() == 0:
+                continue
+            gu = F.linear(h[rows], exp_gu[e]).float() * wts[rows, k:k + 1]
+            g = gu[:, :ff]
+            act = (g * torch.sigmoid(g) * gu[:, ff:]).to(h.dtype)
+            out[rows] += F.linear(act, exp_down[e]).float()
+    return out
