@@ -3,7 +3,8 @@
 #include <vector>
 
 std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
-                                          double eps, bool out_bf16, double offset);
+                                          double eps, bool out_bf16, double offset,
+                                          int64_t groups);
 void gated_residual_add(torch::Tensor x, torch::Tensor mix,
                         c10::optional<torch::Tensor> ff, torch::Tensor gates,
                         torch::Tensor gate_b, double mult);
@@ -48,9 +49,28 @@ torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tail
                             torch::Tensor cu, torch::Tensor tok_seq, torch::Tensor slots,
                             bool out_bf16);
 c10::optional<torch::Tensor> sandwich_residual_norm(
-    torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2, torch::Tensor post_w,
-    c10::optional<torch::Tensor> next_w, double eps, bool out_bf16, double offset,
-    double y_scale, double y2_scale, bool cast_next);
+    torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2,
+    c10::optional<torch::Tensor> post_w, c10::optional<torch::Tensor> next_w, double eps,
+    bool out_bf16, double offset, double y_scale, double y2_scale, bool cast_next,
+    int64_t groups);
+torch::Tensor gelu_tanh(torch::Tensor x);
+std::vector<torch::Tensor> moe_route_sigmoid(torch::Tensor h, torch::Tensor router_w, int64_t top);
+torch::Tensor moe_experts_scaled_input(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                                       torch::Tensor exp_gu, torch::Tensor exp_down);
+torch::Tensor qk_prepare_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
+                                  int64_t vdim, c10::optional<torch::Tensor> q_norm_w,
+                                  c10::optional<torch::Tensor> k_norm_w, double eps,
+                                  torch::Tensor positions, c10::optional<torch::Tensor> freqs,
+                                  double mag, c10::optional<torch::Tensor> mix,
+                                  torch::Tensor page_slot, torch::Tensor cache);
+torch::Tensor window_attention(torch::Tensor q, torch::Tensor cache, int64_t heads,
+                               int64_t kv_heads, int64_t dim, int64_t vdim, bool whole_key,
+                               torch::Tensor block_tables, int64_t block_size,
+                               torch::Tensor tok_seq, torch::Tensor positions, double scale,
+                               int64_t window, int64_t keep_first,
+                               c10::optional<torch::Tensor> r1, c10::optional<torch::Tensor> r2,
+                               c10::optional<torch::Tensor> gate,
+                               c10::optional<torch::Tensor> tiles, int64_t max_tile_queries);
 torch::Tensor capped_glu(torch::Tensor gu, double limit);
 torch::Tensor silu_glu(torch::Tensor gu);
 torch::Tensor qk_norm_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_heads, int64_t dim,
@@ -111,4 +131,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sink_attention", &sink_attention,
         "paged GQA with capped scores, sinks and head mixing");
   m.def("gated_delta_rule", &gated_delta_rule, "gated delta rule with per-slot fp32 state");
+  m.def("gelu_tanh", &gelu_tanh, "tanh-form GELU activation");
+  m.def("moe_route_sigmoid", &moe_route_sigmoid, "fp32 router: sigmoid scores, top-k, no renormalisation");
+  m.def("moe_experts_scaled_input", &moe_experts_scaled_input,
+        "grouped-GEMM mixture of SiLU-gated experts whose input carries the routing weight");
+  m.def("qk_prepare_kv_write", &qk_prepare_kv_write,
+        "q/k norm, half rotary, score-mixing fold of the queries, K/V cache write");
+  m.def("window_attention", &window_attention,
+        "paged GQA softmax attention: window with kept first tokens, log distance bias, output gate");
 }

@@ -2,34 +2,40 @@
 // tails (added to its input, or followed by SiLU), the gated
 // parallel-residual update (alone, and fused with the next layer's norm),
 // the sandwich residual update (closing norm of a sublayer, residual sum and
-// the next opening norm in one pass) and the clamped GLU activation. One
-// workgroup per token row for the row-wise ops.
+// the next opening norm in one pass; without a closing norm it is the
+// pre-norm tail), the clamped GLU and tanh-GELU activations. Norms may be
+// taken over equal consecutive groups of the row. One workgroup per token row
+// for the row-wise ops.
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
 #include "seqmix_common.h"
 
 namespace {
 
-// h = x / sqrt(mean(x^2) + eps) * (offset + w); written as fp32 and (if hb)
-// as T. Input rows are ldx apart (a column slice of a wider matrix).
+// h = x / sqrt(mean(x^2) + eps) * (offset + w), the mean over each of ng
+// equal consecutive parts of the row; written as fp32 and (if hb) as T. Input
+// rows are ldx apart (a column slice of a wider matrix).
 template <typename Tin, typename T>
 __global__ __launch_bounds__(256) void offset_rmsnorm_kernel(
     const Tin* __restrict__ x, int64_t ldx, const float* __restrict__ w, float eps,
-    float offset, int D, float* __restrict__ h32, T* __restrict__ hb) {
+    float offset, int D, int ng, float* __restrict__ h32, T* __restrict__ hb) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const Tin* xr = x + row * ldx;
-  float ss = 0.f;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float v = to_f(xr[d]);
-    ss += v * v;
-  }
-  ss = sm_block_sum(ss, red);
-  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float v = to_f(xr[d]) * inv * (offset + w[d]);
-    h32[row * D + d] = v;
-    if (hb != nullptr) hb[row * D + d] = from_f<T>(v);
+  const int n = D / ng;
+  for (int g = 0; g < ng; ++g) {
+    float ss = 0.f;
+    for (int d = g * n + threadIdx.x; d < (g + 1) * n; d += blockDim.x) {
+      const float v = to_f(xr[d]);
+      ss += v * v;
+    }
+    ss = sm_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int d = g * n + threadIdx.x; d < (g + 1) * n; d += blockDim.x) {
+      const float v = to_f(xr[d]) * inv * (offset + w[d]);
+      h32[row * D + d] = v;
+      if (hb != nullptr) hb[row * D + d] = from_f<T>(v);
+    }
   }
 }
 
@@ -142,9 +148,10 @@ __global__ __launch_bounds__(256) void tap_conv_step_kernel(
   out[(int64_t)b * D + d] = from_f<T>(acc);
 }
 
-// x += s / sqrt(mean(s^2) + eps) * (1 + post_w), s = y (+ y2); then, with
-// next_w, h = x / sqrt(mean(x^2) + eps) * (1 + next_w). y and y2 are bf16 or
-// fp32 each (flags), h is T.
+// x += s / sqrt(mean(s^2) + eps) * (1 + post_w), s = y (+ y2), or x += s
+// without post_w; then, with next_w, h = x / sqrt(mean(x^2) + eps) *
+// (1 + next_w), the mean over each of ng equal parts of the row. y and y2 are
+// bf16 or fp32 each (flags), h is T.
 SM_INLINE float ld_any(const void* p, bool is_bf16, int64_t i) {
   return is_bf16 ? __bfloat162float(reinterpret_cast<const bf16_t*>(p)[i])
                  : reinterpret_cast<const float*>(p)[i];
@@ -154,33 +161,63 @@ __global__ __launch_bounds__(256) void sandwich_residual_kernel(
     float* __restrict__ x, const void* __restrict__ y, bool y_bf16,
     const void* __restrict__ y2, bool y2_bf16, const float* __restrict__ post_w,
     const float* __restrict__ next_w, float eps, float offset, float ys, float y2s,
-    int D, T* __restrict__ h) {
+    int D, int ng, T* __restrict__ h) {
   // the closing norm is over s = ys * y (+ y2s * y2); h (when given) gets the
   // next norm of the new row, or, without next_w, the new row itself
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
-  float ss = 0.f;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float s = ys * ld_any(y, y_bf16, row * D + d);
-    if (y2 != nullptr) s += y2s * ld_any(y2, y2_bf16, row * D + d);
-    ss += s * s;
+  float inv = 1.0f;
+  if (post_w != nullptr) {
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      float s = ys * ld_any(y, y_bf16, row * D + d);
+      if (y2 != nullptr) s += y2s * ld_any(y2, y2_bf16, row * D + d);
+      ss += s * s;
+    }
+    ss = sm_block_sum(ss, red);
+    inv = 1.0f / sqrtf(ss / (float)D + eps);
   }
-  ss = sm_block_sum(ss, red);
-  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
   float xx = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float s = ys * ld_any(y, y_bf16, row * D + d);
     if (y2 != nullptr) s += y2s * ld_any(y2, y2_bf16, row * D + d);
-    const float v = x[row * D + d] + s * inv * (offset + post_w[d]);
+    const float v = x[row * D + d] + (post_w != nullptr ? s * inv * (offset + post_w[d]) : s);
     x[row * D + d] = v;
     xx += v * v;
     if (next_w == nullptr && h != nullptr) h[row * D + d] = from_f<T>(v);
   }
   if (next_w == nullptr) return;
-  xx = sm_block_sum(xx, red);   // also orders the row's writes before the re-read
-  const float inv2 = 1.0f / sqrtf(xx / (float)D + eps);
-  for (int d = threadIdx.x; d < D; d += blockDim.x)
-    h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (offset + next_w[d]));
+  if (ng == 1) {
+    xx = sm_block_sum(xx, red);   // also orders the row's writes before the re-read
+    const float inv2 = 1.0f / sqrtf(xx / (float)D + eps);
+    for (int d = threadIdx.x; d < D; d += blockDim.x)
+      h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (offset + next_w[d]));
+    return;
+  }
+  // grouped norm: another thread may have written what this one reads now
+  __syncthreads();
+  const int n = D / ng;
+  for (int g = 0; g < ng; ++g) {
+    float gs = 0.f;
+    for (int d = g * n + threadIdx.x; d < (g + 1) * n; d += blockDim.x) {
+      const float v = x[row * D + d];
+      gs += v * v;
+    }
+    gs = sm_block_sum(gs, red);
+    const float inv2 = 1.0f / sqrtf(gs / (float)n + eps);
+    for (int d = g * n + threadIdx.x; d < (g + 1) * n; d += blockDim.x)
+      h[row * D + d] = from_f<T>(x[row * D + d] * inv2 * (offset + next_w[d]));
+  }
+}
+
+// 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), fp32 inside.
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const T* __restrict__ x, int64_t n,
+                                                        T* __restrict__ out) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= n) return;
+  const float z = to_f(x[id]);
+  out[id] = from_f<T>(0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))));
 }
 
 // gu rows = [gate (ff) | up (ff)]: g = min(gate, limit), u = clamp(up, +-limit),
@@ -199,10 +236,12 @@ __global__ __launch_bounds__(256) void capped_glu_kernel(
 }  // namespace
 
 std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
-                                          double eps, bool out_bf16, double offset) {
+                                          double eps, bool out_bf16, double offset,
+                                          int64_t groups) {
   SM_CHECK_CUDA(w); SM_CHECK_F32(w);
   TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1 && w.numel() == x.size(1),
               "offset_rmsnorm: shapes");
+  TORCH_CHECK(groups >= 1 && x.size(1) % groups == 0, "offset_rmsnorm: groups must divide the row");
   const int64_t ldx = x.stride(0);
   const int64_t T = x.size(0);
   const int D = x.size(1);
@@ -214,12 +253,12 @@ std::vector<torch::Tensor> offset_rmsnorm(torch::Tensor x, torch::Tensor w,
   if (x.scalar_type() == at::kBFloat16) {
     offset_rmsnorm_kernel<bf16_t, bf16_t><<<T, 256, 0, stream>>>(
         reinterpret_cast<const bf16_t*>(x.data_ptr()), ldx, w.data_ptr<float>(),
-        (float)eps, (float)offset, D, h32.data_ptr<float>(), hbp);
+        (float)eps, (float)offset, D, (int)groups, h32.data_ptr<float>(), hbp);
   } else {
     SM_CHECK_F32(x);
     offset_rmsnorm_kernel<float, bf16_t><<<T, 256, 0, stream>>>(
         x.data_ptr<float>(), ldx, w.data_ptr<float>(), (float)eps, (float)offset, D,
-        h32.data_ptr<float>(), hbp);
+        (int)groups, h32.data_ptr<float>(), hbp);
   }
   SM_CHECK_LAUNCH();
   return {h32, hb};
@@ -385,9 +424,18 @@ torch::Tensor tap_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor tail
 
 c10::optional<torch::Tensor> sandwich_residual_norm(
     torch::Tensor x, torch::Tensor y, c10::optional<torch::Tensor> y2,
-    torch::Tensor post_w, c10::optional<torch::Tensor> next_w, double eps,
-    bool out_bf16, double offset, double y_scale, double y2_scale, bool cast_next) {
-  SM_CHECK_CUDA(x); SM_CHECK_F32(x); SM_CHECK_CUDA(y); SM_CHECK_CUDA(post_w); SM_CHECK_F32(post_w);
+    c10::optional<torch::Tensor> post_w, c10::optional<torch::Tensor> next_w, double eps,
+    bool out_bf16, double offset, double y_scale, double y2_scale, bool cast_next,
+    int64_t groups) {
+  SM_CHECK_CUDA(x); SM_CHECK_F32(x); SM_CHECK_CUDA(y);
+  const float* pw = nullptr;
+  if (post_w.has_value()) {
+    SM_CHECK_CUDA(*post_w); SM_CHECK_F32(*post_w);
+    TORCH_CHECK(post_w->numel() == x.size(1), "sandwich_residual_norm: closing norm weight");
+    pw = post_w->data_ptr<float>();
+  }
+  TORCH_CHECK(groups >= 1 && x.size(1) % groups == 0,
+              "sandwich_residual_norm: groups must divide the row");
   const int64_t T = x.size(0);
   const int D = x.size(1);
   auto kind = [](const torch::Tensor& t) {
@@ -395,7 +443,7 @@ c10::optional<torch::Tensor> sandwich_residual_norm(
                 "sandwich_residual_norm: addends are bf16 or fp32");
     return t.scalar_type() == at::kBFloat16;
   };
-  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == T && y.size(1) == D && post_w.numel() == D,
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && y.size(0) == T && y.size(1) == D,
               "sandwich_residual_norm: shapes");
   const bool yb = kind(y);
   const void* y2p = nullptr;
@@ -421,13 +469,13 @@ c10::optional<torch::Tensor> sandwich_residual_norm(
   auto stream = at::cuda::getCurrentCUDAStream();
   if (out_bf16)
     sandwich_residual_kernel<bf16_t><<<T, 256, 0, stream>>>(
-        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps,
-        (float)offset, (float)y_scale, (float)y2_scale, D,
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, pw, nw, (float)eps,
+        (float)offset, (float)y_scale, (float)y2_scale, D, (int)groups,
         h.has_value() ? reinterpret_cast<bf16_t*>(h->data_ptr()) : nullptr);
   else
     sandwich_residual_kernel<float><<<T, 256, 0, stream>>>(
-        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, post_w.data_ptr<float>(), nw, (float)eps,
-        (float)offset, (float)y_scale, (float)y2_scale, D,
+        x.data_ptr<float>(), y.data_ptr(), yb, y2p, y2b, pw, nw, (float)eps,
+        (float)offset, (float)y_scale, (float)y2_scale, D, (int)groups,
         h.has_value() ? h->data_ptr<float>() : nullptr);
   SM_CHECK_LAUNCH();
   return h;
@@ -458,3 +506,21 @@ static torch::Tensor glu_impl(torch::Tensor gu, double limit) {
 
 torch::Tensor capped_glu(torch::Tensor gu, double limit) { return glu_impl<false>(gu, limit); }
 torch::Tensor silu_glu(torch::Tensor gu) { return glu_impl<true>(gu, 0.0); }
+
+torch::Tensor gelu_tanh(torch::Tensor x) {
+  SM_CHECK_CUDA(x);
+  auto out = torch::empty_like(x);
+  const int64_t n = x.numel();
+  if (n == 0) return out;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  if (x.scalar_type() == at::kBFloat16)
+    gelu_tanh_kernel<bf16_t><<<SM_CDIV(n, 256), 256, 0, stream>>>(
+        reinterpret_cast<const bf16_t*>(x.data_ptr()), n, reinterpret_cast<bf16_t*>(out.data_ptr()));
+  else {
+    SM_CHECK_F32(x);
+    gelu_tanh_kernel<float><<<SM_CDIV(n, 256), 256, 0, stream>>>(x.data_ptr<float>(), n,
+                                                                 out.data_ptr<float>());
+  }
+  SM_CHECK_LAUNCH();
+  return out;
+}

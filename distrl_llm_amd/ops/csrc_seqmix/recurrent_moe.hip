@@ -1,10 +1,13 @@
 // minGRU scan over a flat varlen batch (fp32 state per slot), the fp32
-// top-k routers (softmax over the chosen logits; or softmax over every
-// output with a choice correction and scaled, unnormalised weights), and the
+// top-k routers (softmax over the chosen logits; softmax over every output
+// with a choice correction and scaled, unnormalised weights; or plain sigmoid
+// scores), and the
 // mixture-of-experts feed-forward as two grouped GEMMs over expert-sorted
 // rows (bf16: MFMA 16x16x32 tiles; fp32: plain FMA; SiLU-gated or clamped
 // GLU experts) followed by a fixed-order weighted combine, which also adds
-// the identity experts' share of the input.
+// the identity experts' share of the input. The routing weight multiplies an
+// expert's output (in the combine) or, for designs that scale the expert's
+// input, its gate and up products before the activation.
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
 #include "seqmix_common.h"
@@ -121,13 +124,14 @@ __global__ __launch_bounds__(256) void mingru_chunk_apply_kernel(
 // takes the softmax over the chosen logits.
 // ALL: scores s = softmax over all E outputs (no bias); the top-k of
 // s + corr are chosen; weights = s[chosen] * wscale, not renormalised.
+// sig (not ALL): weights = sigmoid of the chosen logits, not renormalised.
 #define SM_MAX_EXPERTS 256
 template <typename T, bool ALL>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ w,
     const float* __restrict__ bias, int D, int E, int top,
     int* __restrict__ idx, float* __restrict__ wts,
-    const float* __restrict__ corr, float wscale) {
+    const float* __restrict__ corr, float wscale, bool sig) {
   __shared__ float z[SM_MAX_EXPERTS];
   __shared__ float sc[SM_MAX_EXPERTS];
   const int64_t t = blockIdx.x;
@@ -181,13 +185,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
         if (z[e] > bv) { bv = z[e]; best = e; }
       if (best < 0) best = 0;             // all NaN/-inf: keep the write in range
       if (k == 0) vmax = bv;
-      const float p = expf(bv - vmax);
+      const float p = sig ? sm_sigmoid(bv) : expf(bv - vmax);
       idx[t * top + k] = best;
       wts[t * top + k] = p;
       sum += p;
       z[best] = -INFINITY;
     }
-    for (int k = 0; k < top; ++k) wts[t * top + k] /= sum;
+    if (!sig)
+      for (int k = 0; k < top; ++k) wts[t * top + k] /= sum;
   }
 }
 
@@ -196,10 +201,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 // The order inside an expert is arbitrary; every row's result is independent
 // of it and the combine reads rows back through inv. Called with E = weight
 // sets + 1: indices at or above the weight sets (identity experts) share the
-// last bin, whose rows no GEMM touches.
+// last bin, whose rows no GEMM touches. With rw: rw[row] = the pair's routing
+// weight (for experts whose input is scaled).
 __global__ __launch_bounds__(1024) void moe_group_kernel(
     const int* __restrict__ idx, int M, int top, int E, int* __restrict__ off,
-    int* __restrict__ src, int* __restrict__ inv) {
+    int* __restrict__ src, int* __restrict__ inv, const float* __restrict__ wts,
+    float* __restrict__ rw) {
   __shared__ int cnt[SM_MAX_EXPERTS + 1];
   __shared__ int start[SM_MAX_EXPERTS + 2];
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
@@ -224,6 +231,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(
     const int row = start[e] + atomicAdd(&cnt[e], 1);
     src[row] = i / top;
     inv[i] = row;
+    if (rw != nullptr) rw[row] = wts[i];
   }
 }
 
@@ -233,6 +241,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(
 // wave w owns columns w*16..w*16+15 for the four 16-row m-tiles.
 // MODE 0: out[i, f] = act(a_i . Wg[f], a_i . Wu[f]), a_i = A[src[i]],
 //         act(g, u) = silu(g) u (limit 0) or the clamped GLU (limit > 0);
+//         with rw both products are scaled by rw[i] first (W (w a) = w (W a));
 //         W[e] = [gate (N rows); up (N rows)] x K;   out bf16 [M, N]
 // MODE 1: out[i, n] = a_i . W[e][n], a_i = A[i];     out fp32 [M, N]
 // MFMA 16x16x32 bf16 fragments: A lane l -> row l&15, k (l>>4)*8..+7;
@@ -262,7 +271,7 @@ template <int MODE, int MT, int NWV>
 __global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const int* __restrict__ src,
     const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
-    int K, void* __restrict__ outp, float limit) {
+    int K, void* __restrict__ outp, float limit, const float* __restrict__ rw) {
   constexpr int BM = 16 * MT;
   __shared__ __attribute__((aligned(16))) bf16_t a_lds[BM * GG_LD];
   // which expert / row range is this tile?
@@ -334,8 +343,9 @@ __global__ __launch_bounds__(64 * NWV) void moe_gemm_bf16_kernel(
       if (r < rows) {
         const int64_t o = (int64_t)(row0 + r) * N + n;
         if (MODE == 0) {
+          const float w = (rw != nullptr) ? rw[row0 + r] : 1.0f;
           reinterpret_cast<bf16_t*>(outp)[o] =
-              __float2bfloat16(moe_act(acc[mt][rr], acc2[mt][rr], limit));
+              __float2bfloat16(moe_act(w * acc[mt][rr], w * acc2[mt][rr], limit));
         } else {
           reinterpret_cast<float*>(outp)[o] = acc[mt][rr];
         }
@@ -353,7 +363,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_splitk_kernel(
     const bf16_t* __restrict__ A, const int* __restrict__ src,
     const bf16_t* __restrict__ W, const int* __restrict__ off, int E, int N,
-    int K, void* __restrict__ outp, float limit) {
+    int K, void* __restrict__ outp, float limit, const float* __restrict__ rw) {
   __shared__ float red[3][64][8];
   int e = -1, row0 = 0, rows = 0, tiles = 0;
   for (int i = 0; i < E; ++i) {
@@ -410,9 +420,10 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_splitk_kernel(
     const int r = lk * 4 + rr;
     if (r < rows) {
       const int64_t o = (int64_t)(row0 + r) * N + n;
-      if (MODE == 0)
-        reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(moe_act(g, u, limit));
-      else
+      if (MODE == 0) {
+        const float w = (rw != nullptr) ? rw[row0 + r] : 1.0f;
+        reinterpret_cast<bf16_t*>(outp)[o] = __float2bfloat16(moe_act(w * g, w * u, limit));
+      } else
         reinterpret_cast<float*>(outp)[o] = g;
     }
   }
@@ -424,7 +435,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
     const float* __restrict__ A, const int* __restrict__ src,
     const float* __restrict__ W, const int* __restrict__ off, int E, int M,
-    int N, int K, float* __restrict__ out, float limit) {
+    int N, int K, float* __restrict__ out, float limit, const float* __restrict__ rw) {
   const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= (int64_t)M * N) return;
   const int i = id / N, n = id % N;
@@ -439,11 +450,13 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
     g = fmaf(a[k], wg[k], g);
     if (MODE == 0) u = fmaf(a[k], wg[(int64_t)N * K + k], u);
   }
+  if (MODE == 0 && rw != nullptr) { g *= rw[i]; u *= rw[i]; }
   out[id] = (MODE == 0) ? moe_act(g, u, limit) : g;
 }
 
-// out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order); a
-// choice at or above E is an identity expert: its output is the input row.
+// out[t, d] = sum_k wts[t, k] * y[inv[t * top + k], d]   (k in order; wts
+// null: every weight is 1); a choice at or above E is an identity expert: its
+// output is the input row.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const float* __restrict__ y, const int* __restrict__ inv,
@@ -455,7 +468,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
     for (int k = 0; k < top; ++k) {
       const float v = (idx[t * top + k] >= E) ? to_f(h[t * D + d])
                                               : y[(int64_t)inv[t * top + k] * D + d];
-      acc += wts[t * top + k] * v;
+      acc += (wts != nullptr ? wts[t * top + k] : 1.0f) * v;
     }
     out[t * D + d] = acc;
   }
@@ -531,7 +544,8 @@ torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bias, torch::Tensor s
 
 static std::vector<torch::Tensor> moe_route_impl(
     torch::Tensor h, torch::Tensor router_w, c10::optional<torch::Tensor> router_b,
-    int64_t top, bool all, c10::optional<torch::Tensor> corr, double wscale) {
+    int64_t top, bool all, c10::optional<torch::Tensor> corr, double wscale,
+    bool sig = false) {
   SM_CHECK_CUDA(h); SM_CHECK_CUDA(router_w); SM_CHECK_F32(router_w);
   const int64_t T = h.size(0);
   const int D = h.size(1);
@@ -559,7 +573,7 @@ static std::vector<torch::Tensor> moe_route_impl(
 #define ROUTE(TY, ALLV)                                                                    \
   moe_route_kernel<TY, ALLV><<<T, 256, 0, stream>>>(                                       \
       reinterpret_cast<const TY*>(h.data_ptr()), router_w.data_ptr<float>(), bp, D, E,     \
-      (int)top, idx.data_ptr<int>(), wts.data_ptr<float>(), cp, (float)wscale)
+      (int)top, idx.data_ptr<int>(), wts.data_ptr<float>(), cp, (float)wscale, sig)
   if (bf16) { if (all) ROUTE(bf16_t, true); else ROUTE(bf16_t, false); }
   else { if (all) ROUTE(float, true); else ROUTE(float, false); }
 #undef ROUTE
@@ -578,8 +592,14 @@ std::vector<torch::Tensor> moe_route_all(torch::Tensor h, torch::Tensor router_w
   return moe_route_impl(h, router_w, c10::nullopt, top, true, correction, scale);
 }
 
+std::vector<torch::Tensor> moe_route_sigmoid(torch::Tensor h, torch::Tensor router_w,
+                                             int64_t top) {
+  return moe_route_impl(h, router_w, c10::nullopt, top, false, c10::nullopt, 1.0, true);
+}
+
 static torch::Tensor moe_experts_impl(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
-                                      torch::Tensor exp_gu, torch::Tensor exp_down, float limit) {
+                                      torch::Tensor exp_gu, torch::Tensor exp_down, float limit,
+                                      bool scale_input = false) {
   SM_CHECK_CUDA(h); SM_CHECK_CUDA(idx); SM_CHECK_I32(idx); SM_CHECK_CUDA(wts); SM_CHECK_F32(wts);
   SM_CHECK_CUDA(exp_gu); SM_CHECK_CUDA(exp_down);
   const int64_t T = h.size(0);
@@ -603,9 +623,16 @@ static torch::Tensor moe_experts_impl(torch::Tensor h, torch::Tensor idx, torch:
   auto src = torch::empty({M}, iopt);
   auto inv = torch::empty({M}, iopt);
   auto stream = at::cuda::getCurrentCUDAStream();
+  torch::Tensor row_w;
+  const float* rw = nullptr;
+  if (scale_input) {
+    row_w = torch::empty({M}, wts.options());
+    rw = row_w.data_ptr<float>();
+  }
   moe_group_kernel<<<1, 1024, 0, stream>>>(idx.data_ptr<int>(), (int)M, top, E + 1,
                                            off.data_ptr<int>(), src.data_ptr<int>(),
-                                           inv.data_ptr<int>());
+                                           inv.data_ptr<int>(), wts.data_ptr<float>(),
+                                           scale_input ? row_w.data_ptr<float>() : nullptr);
   SM_CHECK_LAUNCH();
   auto y = torch::empty({M, D}, out.options());
   if (h.scalar_type() == at::kBFloat16) {
@@ -617,20 +644,20 @@ static torch::Tensor moe_experts_impl(torch::Tensor h, torch::Tensor idx, torch:
       // a few rows per expert (decoding): 16x16 tiles, K split over four waves
       const int row_tiles = SM_CDIV(M, 16) + E;
       moe_gemm_bf16_splitk_kernel<0><<<dim3(row_tiles, SM_CDIV(ff, 16)), 256, 0, stream>>>(
-          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit);
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit, rw);
       SM_CHECK_LAUNCH();
       moe_gemm_bf16_splitk_kernel<1><<<dim3(row_tiles, SM_CDIV(D, 16)), 256, 0, stream>>>(
           reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
-          D, ff, y.data_ptr(), 0.f);
+          D, ff, y.data_ptr(), 0.f, nullptr);
       SM_CHECK_LAUNCH();
     } else {
       const int row_tiles = SM_CDIV(M, 64) + E;
       moe_gemm_bf16_kernel<0, 4, 4><<<dim3(row_tiles, SM_CDIV(ff, 64)), 256, 0, stream>>>(
-          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit);
+          hp, src.data_ptr<int>(), gup, off.data_ptr<int>(), E, ff, D, act.data_ptr(), limit, rw);
       SM_CHECK_LAUNCH();
       moe_gemm_bf16_kernel<1, 4, 4><<<dim3(row_tiles, SM_CDIV(D, 64)), 256, 0, stream>>>(
           reinterpret_cast<const bf16_t*>(act.data_ptr()), nullptr, dnp, off.data_ptr<int>(), E,
-          D, ff, y.data_ptr(), 0.f);
+          D, ff, y.data_ptr(), 0.f, nullptr);
       SM_CHECK_LAUNCH();
     }
   } else {
@@ -638,21 +665,22 @@ static torch::Tensor moe_experts_impl(torch::Tensor h, torch::Tensor idx, torch:
     auto act = torch::empty({M, ff}, h.options());
     moe_gemm_f32_kernel<0><<<SM_CDIV(M * ff, 256), 256, 0, stream>>>(
         h.data_ptr<float>(), src.data_ptr<int>(), exp_gu.data_ptr<float>(),
-        off.data_ptr<int>(), E, (int)M, ff, D, act.data_ptr<float>(), limit);
+        off.data_ptr<int>(), E, (int)M, ff, D, act.data_ptr<float>(), limit, rw);
     SM_CHECK_LAUNCH();
     moe_gemm_f32_kernel<1><<<SM_CDIV(M * D, 256), 256, 0, stream>>>(
         act.data_ptr<float>(), nullptr, exp_down.data_ptr<float>(), off.data_ptr<int>(), E,
-        (int)M, D, ff, y.data_ptr<float>(), 0.f);
+        (int)M, D, ff, y.data_ptr<float>(), 0.f, nullptr);
     SM_CHECK_LAUNCH();
   }
   if (h.scalar_type() == at::kBFloat16)
     moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>(
-        y.data_ptr<float>(), inv.data_ptr<int>(), wts.data_ptr<float>(), idx.data_ptr<int>(),
-        reinterpret_cast<const bf16_t*>(h.data_ptr()), E, top, D, out.data_ptr<float>());
+        y.data_ptr<float>(), inv.data_ptr<int>(), scale_input ? nullptr : wts.data_ptr<float>(),
+        idx.data_ptr<int>(), reinterpret_cast<const bf16_t*>(h.data_ptr()), E, top, D,
+        out.data_ptr<float>());
   else
     moe_combine_kernel<float><<<T, 256, 0, stream>>>(
-        y.data_ptr<float>(), inv.data_ptr<int>(), wts.data_ptr<float>(), idx.data_ptr<int>(),
-        h.data_ptr<float>(), E, top, D, out.data_ptr<float>());
+        y.data_ptr<float>(), inv.data_ptr<int>(), scale_input ? nullptr : wts.data_ptr<float>(),
+        idx.data_ptr<int>(), h.data_ptr<float>(), E, top, D, out.data_ptr<float>());
   SM_CHECK_LAUNCH();
   return out;
 }
@@ -666,4 +694,9 @@ torch::Tensor moe_experts_glu(torch::Tensor h, torch::Tensor idx, torch::Tensor 
                               torch::Tensor exp_gu, torch::Tensor exp_down, double limit) {
   TORCH_CHECK(limit > 0, "moe_experts_glu: the clamp limit must be positive");
   return moe_experts_impl(h, idx, wts, exp_gu, exp_down, (float)limit);
+}
+
+torch::Tensor moe_experts_scaled_input(torch::Tensor h, torch::Tensor idx, torch::Tensor wts,
+                                       torch::Tensor exp_gu, torch::Tensor exp_down) {
+  return moe_experts_impl(h, idx, wts, exp_gu, exp_down, 0.f, true);
 }
