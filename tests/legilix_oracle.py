@@ -194,3 +194,90 @@ def forward(cfg, w, tokens, layers_out=None):
             layers_out.append(x.clone())
     x = group_norm(x, w["final.norm"].to(F64), groups, eps)
     return (x @ E.t()) * float(cfg["logit_scale"])
+
+
+# ------------------------------------------------- small configs for tests
+
+def rotary_layer(heads=4, kv_heads=2, dim=8, vdim=6, window=7, keep=2, rot_dims=4,
+                 base=100.0, scaling=(4.0, 16, 2.0, 0.5), scale=None, mlp=12):
+    """An 'attention' layer; ``mlp`` an int (dense ff), a tuple (experts,
+    top, ff) or None."""
+    rot = {"base": base, "dims": rot_dims}
+    if scaling:
+        rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    mask = {"size": window, "keep_first": keep} if window else {}
+    mc = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+          "mask": mask, "rot": rot, "scale": scale if scale is not None else dim ** -0.5}
+    return {"type": "attention", "mixer": mc, "mlp": _mlp(mlp)}
+
+
+def distance_layer(heads=4, kv_heads=2, dim=8, vdim=6, window=7, scale=None, mlp=12):
+    """An 'attention_2' layer."""
+    mc = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+          "mask": {"size": window} if window else {},
+          "scale": scale if scale is not None else dim ** -0.5}
+    return {"type": "attention_2", "mixer": mc, "mlp": _mlp(mlp)}
+
+
+def _mlp(m):
+    if m is None:
+        return None
+    if isinstance(m, int):
+        return {"kind": "dense", "ff": m}
+    experts, top, ff = m
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def make_cfg(layers, width=24, vocab=37, groups=3, eps=1e-5, embed_scale=3.0,
+             logit_scale=0.5):
+    return {"architecture": "Legilix", "embedding": {"scale": embed_scale},
+            "layers": layers, "logit_scale": logit_scale,
+            "norm": {"eps": eps, "groups": groups}, "vocab": vocab, "width": width}
+
+
+def random_weights(cfg, seed=0):
+    """Checkpoint tensors of a configuration, rounded to bfloat16 as a
+    checkpoint file holds them."""
+    g = torch.Generator().manual_seed(seed)
+    D = int(cfg["width"])
+    w = {}
+
+    def mat(name, rows, cols):
+        w[name] = torch.randn(rows, cols, generator=g) / math.sqrt(cols)
+
+    def vec(name, n, mean=0.0, std=0.1):
+        w[name] = mean + std * torch.randn(n, generator=g)
+
+    w["embed"] = torch.randn(int(cfg["vocab"]), D, generator=g) * 0.5
+    vec("final.norm", D, 1.0)
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc = f"l{i}.", lc["mixer"]
+        H, G, dk, dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        vec(p + "norm1", D, 1.0)
+        for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+            mat(p + "mix." + nm, rows, D)
+            vec(p + "mix." + nm + ".b", rows, 0.0, 0.3)
+        if lc["type"] == "attention":
+            vec(p + "mix.q.norm", dk, 1.0, 0.2)
+            vec(p + "mix.k.norm", dk, 1.0, 0.2)
+            w[p + "mix.talk"] = torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)
+        else:
+            vec(p + "mix.r1", H, 0.6, 0.3)
+            w[p + "mix.r2"] = 0.2 + torch.rand(H, generator=g)
+            mat(p + "mix.g", H, D)
+        mat(p + "mix.o", D, H * dv)
+        fc = lc.get("mlp")
+        if fc is None:
+            continue
+        vec(p + "norm2", D, 1.0)
+        if fc["kind"] == "dense":
+            mat(p + "mlp.up", fc["ff"], D)
+            mat(p + "mlp.down", D, fc["ff"])
+        else:
+            ff = fc["expert"]["ff"]
+            mat(p + "mlp.router", fc["router"]["experts"], D)
+            for e in range(fc["router"]["experts"]):
+                mat(f"{p}mlp.e{e}.gate", ff, D)
+                mat(f"{p}mlp.e{e}.up", ff, D)
+                mat(f"{p}mlp.e{e}.down", D, ff)
+    return {k: v.to(torch.bfloat16).float() for k, v in w.items()}
