@@ -51,12 +51,13 @@ def parse_args():
                         "no-EOS rounds). Measures in-wave retirement.")
     p.add_argument("--hybrid-bench", type=str, default="",
                    help="instead of the RL round: prefill/decode tokens/s of "
-                        "the layer-list designs (Kakilorn, Nedasun, Nibalix) beside the "
+                        "the layer-list designs (Legilix, Kakilorn, Nedasun, Nibalix) beside the "
                         "dense model of equal size, at these comma-separated "
                         "sizes (1k,2k)")
     p.add_argument("--hybrid-only", type=str, default="",
-                   help="with --hybrid-bench: run only these of 'kakilorn', "
-                        "'nedasun', 'nibalix', 'dense' (comma-separated)")
+                   help="with --hybrid-bench: run only these of 'legilix', "
+                        "'kakilorn', 'nedasun', 'nibalix', 'dense' "
+                        "(comma-separated)")
     p.add_argument("--tiny", action="store_true",
                    help="tiny model + short generations (debug only; NOT the "
                         "headline config)")
@@ -70,7 +71,7 @@ def main():
         dev = torch.device("cuda:0" if torch.cuda.is_available() and not args.cpu
                            else "cpu")
         which = (tuple(args.hybrid_only.split(",")) if args.hybrid_only
-                 else ("kakilorn", "nedasun", "nibalix", "dense"))
+                 else ("legilix", "kakilorn", "nedasun", "nibalix", "dense"))
         bench_hybrid.run(args.hybrid_bench.split(","), dev, which=which)
         return
     rank = int(os.environ.get("RANK", "0"))

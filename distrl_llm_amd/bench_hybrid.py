@@ -1,5 +1,5 @@
 """Prefill and decode throughput of the layer-list designs (Nibalix,
-Nedasun, Kakilorn) beside one another and beside the dense transformer of equal size
+Nedasun, Kakilorn, Legilix) beside one another and beside the dense transformer of equal size
 (``bench.py --hybrid-bench``).
 
 All models get random weights at layer sizes that resemble a real model
@@ -11,6 +11,7 @@ generation.
 
 from __future__ import annotations
 
+import gc
 import json
 import time
 
@@ -115,12 +116,47 @@ def kakilorn_bench_config(s: dict) -> dict:
             "vocab": s["vocab"], "width": s["width"]}
 
 
+def legilix_bench_config(s: dict) -> dict:
+    """Same width, depth, head count and head sizes (128/128, 4 query heads
+    per kv head) as the Nedasun config of the size; every layer is windowed
+    attention: the distance-bias form and the rotary form with mixed scores
+    alternate (window of the size, 16 kept tokens), feed-forwards alternate
+    between the experts of the other designs and a dense MLP as wide as the
+    experts one token uses; norms over four groups."""
+    kvh = max(1, s["heads"] // 4)
+    moe = {"kind": "moe", "expert": {"ff": s["ff"]},
+           "router": {"experts": s["experts"], "top": s["top"]}}
+    dense = {"kind": "dense", "ff": s["top"] * s["ff"]}
+    base = {"heads": s["heads"], "kv_heads": kvh, "dim": 128, "vdim": 128,
+            "scale": 128 ** -0.5}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            mc = dict(base, mask={"size": s["window"]})
+            layers.append({"type": "attention_2", "mixer": mc,
+                           "mlp": dense if i % 4 == 0 else moe})
+        else:
+            mc = dict(base, mask={"size": s["window"], "keep_first": 16},
+                      rot={"base": 10000.0, "dims": 64,
+                           "scaling": {"factor": 4.0, "original": 4096,
+                                       "fast": 32.0, "slow": 1.0}})
+            layers.append({"type": "attention", "mixer": mc,
+                           "mlp": moe if i % 4 == 1 else dense})
+    return {"architecture": "Legilix", "embedding": {"scale": 1.0},
+            "layers": layers, "logit_scale": 1.0,
+            "norm": {"eps": 1e-5, "groups": 4}, "vocab": s["vocab"],
+            "width": s["width"]}
+
+
 def _build_hybrid(s, device, max_len, batch, design="nibalix"):
     from .engine.hybrid_engine import HybridEngine
     from .models.hybrid import (HybridLM, kakilorn_spec_from_config,
+                                legilix_spec_from_config,
                                 nedasun_spec_from_config,
                                 nibalix_spec_from_config)
-    if design == "kakilorn":
+    if design == "legilix":
+        spec = legilix_spec_from_config(legilix_bench_config(s))
+    elif design == "kakilorn":
         spec = kakilorn_spec_from_config(kakilorn_bench_config(s))
     elif design == "nedasun":
         spec = nedasun_spec_from_config(nedasun_bench_config(s))
@@ -172,7 +208,7 @@ def measure(engine, vocab, batch, prompt_len, new_tokens, device):
             "prefill_s": t_pre, "decode_ms_per_step": 1e3 * dec / (new_tokens - 1)}
 
 
-def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("kakilorn", "nedasun", "nibalix", "dense")):
+def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("legilix", "kakilorn", "nedasun", "nibalix", "dense")):
     out = []
     for name in sizes:
         s = SIZES[name]
@@ -189,6 +225,7 @@ def run(sizes, device, batch=16, prompt_len=1024, new_tokens=33, which=("kakilor
             print(json.dumps(line), flush=True)
             out.append(line)
             del eng
+            gc.collect()        # the engine and its captured steps are a cycle
             if device.type == "cuda":
                 torch.cuda.empty_cache()
     return out

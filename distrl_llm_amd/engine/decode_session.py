@@ -29,6 +29,7 @@ from typing import List, Optional
 import torch
 
 from ..config import SamplingParams
+from ..utils.capture import collector_paused
 from .kvcache import KVCachePool, Sequence
 
 
@@ -149,7 +150,7 @@ class DecodeSession:
         for t, sv in zip(state, saved):
             t.copy_(sv)
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with collector_paused(), torch.cuda.graph(g):
             self._step()
         self.graph = g
 

@@ -30,6 +30,7 @@ from ..models.hybrid import (DeltaRuleSpec, GluSpec, HybridLM,
                              WindowAttentionSpec)
 from ..ops import functional as OF
 from ..ops import seqmix as SM
+from ..utils.capture import collector_paused
 from ..utils.trace import trace_range
 from .kvcache import Sequence
 from .seqstate import LatentCachePool, StateSlotPool
@@ -62,7 +63,7 @@ class _DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with collector_paused(), torch.cuda.graph(self.graph):
             self.logits = self._body()
 
     def _flat(self, tokens, positions, page_slot, slots, tables):
