@@ -28,6 +28,24 @@ SM_INLINE float sm_wave_max(float x) {
   for (int off = 32; off > 0; off >>= 1) x = fmaxf(x, __shfl_xor(x, off, SM_WAVE));
   return x;
 }
+// Reductions over the 16 lanes of a row (lanes that share lane >> 4) on the
+// VALU's lane-permute path: the two quad swaps, then the mirrors of 8 and of
+// 16 lanes; afterwards every lane of the row holds the result.
+template <int CTRL> SM_INLINE float sm_dpp(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+SM_INLINE float sm_row16_max(float x) {
+  x = fmaxf(x, sm_dpp<0xB1>(x));    // quad_perm [1, 0, 3, 2]
+  x = fmaxf(x, sm_dpp<0x4E>(x));    // quad_perm [2, 3, 0, 1]
+  x = fmaxf(x, sm_dpp<0x141>(x));   // row_half_mirror
+  return fmaxf(x, sm_dpp<0x140>(x));   // row_mirror
+}
+SM_INLINE float sm_row16_sum(float x) {
+  x += sm_dpp<0xB1>(x);
+  x += sm_dpp<0x4E>(x);
+  x += sm_dpp<0x141>(x);
+  return x + sm_dpp<0x140>(x);
+}
 // Sum over a block of up to 1024 threads; red needs blockDim.x / 64 floats.
 SM_INLINE float sm_block_sum(float x, float* red) {
   const int lane = threadIdx.x & (SM_WAVE - 1), wid = threadIdx.x / SM_WAVE;

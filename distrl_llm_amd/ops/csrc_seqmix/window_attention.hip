@@ -24,70 +24,113 @@
 
 namespace {
 
+// Two neighbouring outputs as one store (the caller checks evenness).
+SM_INLINE void wa_store2(float* p, float a, float b) {
+  *reinterpret_cast<float2*>(p) = make_float2(a, b);
+}
+SM_INLINE void wa_store2(bf16_t* p, float a, float b) {
+  const unsigned int lo = __bfloat16_as_ushort(__float2bfloat16(a));
+  const unsigned int hi = __bfloat16_as_ushort(__float2bfloat16(b));
+  *reinterpret_cast<unsigned int*>(p) = lo | (hi << 16);
+}
+
 // One workgroup per token. proj row = [q (H dk) | k (G dk) | v (G vd) | ...],
-// rows ldp apart. The H + G heads pass through LDS as fp32: norm (a wave per
-// head), rotation of entries (i, i + half) by p * freqs[i] with cos and sin
-// times mag, then k -> cache row, v -> cache row, and q -> q_out [H, dk], or
-// with mix (fp32 [H, H]) the folded queries [H, G dk].
-template <typename T>
+// rows ldp apart. The H + G heads pass through LDS as fp32: the whole row is
+// fetched at once, then a wave per head norms it and rotates entries
+// (i, i + half) by p * freqs[i] with cos and sin times mag (one sincos per
+// pair and token, shared by the heads); then k -> cache row, v -> cache row,
+// and q -> q_out [H, dk], or with mix (fp32 [H, H]) the folded queries
+// [H, G dk]. PAIR: dk and vd are even and rows start on 4-byte borders, so
+// outputs go out two at a time.
+template <typename T, bool PAIR>
 __global__ __launch_bounds__(256) void qk_prepare_kv_write_kernel(
     const T* __restrict__ proj, int64_t ldp, int H, int G, int dk, int vd,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps,
     const int* __restrict__ positions, const float* __restrict__ freqs, int half, float mag,
     const float* __restrict__ mix, const int* __restrict__ page_slot, T* __restrict__ cache,
     T* __restrict__ q_out) {
-  extern __shared__ float hb[];                      // [(H + G) dk]
+  extern __shared__ float hb[];                      // [(H + G) dk] | cos, sin [2 half] | mix [H H]
+  const int nqk = (H + G) * dk;
+  float* cs = hb + nqk;
+  float* mx = cs + 2 * half;
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = proj + t * ldp;
-  for (int job = wave; job < H + G; job += 4) {
-    const T* src = row + (int64_t)job * dk;          // q heads, then k heads
-    float inv = 1.0f;
-    const float* w = nullptr;
-    if (qw != nullptr) {
-      float ss = 0.f;
-      for (int k = lane; k < dk; k += 64) {
-        const float v = to_f(src[k]);
-        ss += v * v;
-      }
-      ss = sm_wave_sum(ss);
-      inv = 1.0f / sqrtf(ss / (float)dk + eps);
-      w = (job >= H) ? kw : qw;
-    }
-    for (int k = lane; k < dk; k += 64)
-      hb[job * dk + k] = (w != nullptr) ? to_f(src[k]) * inv * w[k] : to_f(src[k]);
+  for (int i = threadIdx.x; i < nqk; i += blockDim.x) hb[i] = to_f(row[i]);
+  if ((int)threadIdx.x < half) {
+    float s, c;
+    sincosf((float)positions[t] * freqs[threadIdx.x], &s, &c);
+    cs[threadIdx.x] = c * mag;
+    cs[half + threadIdx.x] = s * mag;
   }
+  if (mix != nullptr)
+    for (int i = threadIdx.x; i < H * H; i += blockDim.x) mx[i] = mix[i];
   __syncthreads();
-  if (half > 0) {
-    const float p = (float)positions[t];
-    for (int i = threadIdx.x; i < (H + G) * half; i += blockDim.x) {
-      const int job = i / half, pi = i % half;
-      float s, c;
-      sincosf(p * freqs[pi], &s, &c);
-      s *= mag;
-      c *= mag;
-      float* e = hb + job * dk + pi;
-      const float a = e[0], b = e[half];
-      e[0] = a * c - b * s;
-      e[half] = b * c + a * s;
+  if (qw != nullptr || half > 0) {
+    for (int job = wave; job < H + G; job += 4) {    // q heads, then k heads
+      float* e = hb + job * dk;
+      if (qw != nullptr) {
+        float ss = 0.f;
+        for (int k = lane; k < dk; k += 64) ss += e[k] * e[k];
+        ss = sm_wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)dk + eps);
+        const float* w = (job >= H) ? kw : qw;
+        for (int k = lane; k < dk; k += 64) e[k] = e[k] * inv * w[k];
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);          // the wave's LDS writes have landed
+      }
+      for (int pi = lane; pi < half; pi += 64) {
+        const float c = cs[pi], sn = cs[half + pi];
+        const float a = e[pi], b = e[pi + half];
+        e[pi] = a * c - b * sn;
+        e[pi + half] = b * c + a * sn;
+      }
     }
     __syncthreads();
   }
   const int nk = G * dk, nv = G * vd;
   T* dst = cache + (int64_t)page_slot[t] * (nk + nv);
+  const T* v = row + nqk;
+  const int rep = H / G;
+  if (PAIR) {
+    for (int i = 2 * threadIdx.x; i < nk; i += 2 * blockDim.x)
+      wa_store2(dst + i, hb[H * dk + i], hb[H * dk + i + 1]);
+    for (int i = 2 * threadIdx.x; i < nv; i += 2 * blockDim.x)
+      wa_store2(dst + nk + i, to_f(v[i]), to_f(v[i + 1]));
+    if (mix == nullptr) {
+      for (int i = 2 * threadIdx.x; i < H * dk; i += 2 * blockDim.x)
+        wa_store2(q_out + t * H * dk + i, hb[i], hb[i + 1]);
+      return;
+    }
+    for (int hc = wave; hc < H * G; hc += 4) {       // (output head, kv head) per wave
+      const int h = hc / G, c = hc % G;
+      const float* m = mx + h * H + c * rep;
+      const float* src = hb + c * rep * dk;
+      T* o = q_out + (t * H + h) * nk + c * dk;
+      for (int k = 2 * lane; k < dk; k += 128) {
+        float a0 = 0.f, a1 = 0.f;
+        for (int r = 0; r < rep; ++r) {
+          a0 = fmaf(m[r], src[r * dk + k], a0);
+          a1 = fmaf(m[r], src[r * dk + k + 1], a1);
+        }
+        wa_store2(o + k, a0, a1);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < nk; i += blockDim.x) dst[i] = from_f<T>(hb[H * dk + i]);
-  const T* v = row + (int64_t)(H + G) * dk;
   for (int i = threadIdx.x; i < nv; i += blockDim.x) dst[nk + i] = v[i];
   if (mix == nullptr) {
     for (int i = threadIdx.x; i < H * dk; i += blockDim.x) q_out[t * H * dk + i] = from_f<T>(hb[i]);
     return;
   }
-  const int rep = H / G;
-  for (int i = threadIdx.x; i < H * nk; i += blockDim.x) {
-    const int h = i / nk, c = (i % nk) / dk, k = i % dk;
-    float a = 0.f;
-    for (int r = 0; r < rep; ++r) a = fmaf(mix[h * H + c * rep + r], hb[(c * rep + r) * dk + k], a);
-    q_out[t * H * nk + i] = from_f<T>(a);
+  for (int hc = wave; hc < H * G; hc += 4) {
+    const int h = hc / G, c = hc % G;
+    for (int k = lane; k < dk; k += 64) {
+      float a = 0.f;
+      for (int r = 0; r < rep; ++r) a = fmaf(mx[h * H + c * rep + r], hb[(c * rep + r) * dk + k], a);
+      q_out[(t * H + h) * nk + c * dk + k] = from_f<T>(a);
+    }
   }
 }
 
@@ -174,8 +217,8 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
 // head g, key share z). The REP query heads of g sit in LDS as fp32 (KD
 // entries each); the visible keys are cut into blocks of 64, share z takes a
 // contiguous run of blocks and its waves take them in turn. Per block: lane =
-// key, the key columns are read once in 16-byte pieces and dotted with all REP
-// queries; every wave keeps its own running max and sum per head; the REP x 64
+// key, the key columns are read once in 16-byte pieces (four in flight) and
+// dotted with all REP queries; every wave keeps its own running max and sum per head; the REP x 64
 // weights go through a wave-private LDS tile; then lane = pair of value
 // columns, and every V row is read once for all REP heads. The waves' states
 // are merged in LDS; with ksplit > 1 the workgroup leaves (max, sum, weighted
@@ -266,13 +309,22 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
       j = (i < nfirst) ? i : lo + (i - nfirst);
       row = bt[j / block_size] * block_size + j % block_size;
       const T* kp = cache + (int64_t)row * W + koff;
-      for (int k = 0; k < KD; k += VN) {
-        float kv[VN];
-        wa_vec<T>::load(kp + k, kv);
+      // four 16-byte pieces of the key row in flight before their products
+      for (int k = 0; k < KD; k += 4 * VN) {
+        float kv[4][VN];
         #pragma unroll
-        for (int hh = 0; hh < REP; ++hh)
-          #pragma unroll
-          for (int e = 0; e < VN; ++e) s[hh] = fmaf(qs[hh * KD + k + e], kv[e], s[hh]);
+        for (int u = 0; u < 4; ++u)
+          wa_vec<T>::load(kp + min(k + u * VN, KD - VN), kv[u]);   // past the end: unused
+        #pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int ku = k + u * VN;
+          if (ku < KD) {
+            #pragma unroll
+            for (int hh = 0; hh < REP; ++hh)
+              #pragma unroll
+              for (int e = 0; e < VN; ++e) s[hh] = fmaf(qs[hh * KD + ku + e], kv[u][e], s[hh]);
+          }
+        }
       }
     }
     float corr[REP];
@@ -301,18 +353,29 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
         acc[hh][c][1] *= corr[hh];
       }
     const int nkeys = min(64, n - kb * 64);
-    for (int jj = 0; jj < nkeys; ++jj) {
-      const T* vp = cache + (int64_t)krow[jj] * W + G * dk + g * vd;
+    // eight V rows in flight before their products
+    for (int jj0 = 0; jj0 < nkeys; jj0 += 8) {
+      float2 v[8][WAG_CP];
       #pragma unroll
-      for (int c = 0; c < WAG_CP; ++c) {
-        const int d = 2 * lane + 128 * c;
-        if (d < vd) {
-          const float2 v = wa_vec<T>::load2(vp + d);
+      for (int u = 0; u < 8; ++u) {
+        const T* vp = cache + (int64_t)krow[min(jj0 + u, nkeys - 1)] * W + G * dk + g * vd;
+        #pragma unroll
+        for (int c = 0; c < WAG_CP; ++c) {
+          const int d = 2 * lane + 128 * c;
+          v[u][c] = (d < vd) ? wa_vec<T>::load2(vp + d) : make_float2(0.f, 0.f);
+        }
+      }
+      #pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (jj0 + u < nkeys) {
           #pragma unroll
-          for (int hh = 0; hh < REP; ++hh) {
-            const float w = pw[hh * 64 + jj];
-            acc[hh][c][0] = fmaf(w, v.x, acc[hh][c][0]);
-            acc[hh][c][1] = fmaf(w, v.y, acc[hh][c][1]);
+          for (int c = 0; c < WAG_CP; ++c) {
+            #pragma unroll
+            for (int hh = 0; hh < REP; ++hh) {
+              const float w = pw[hh * 64 + jj0 + u];
+              acc[hh][c][0] = fmaf(w, v[u][c].x, acc[hh][c][0]);
+              acc[hh][c][1] = fmaf(w, v[u][c].y, acc[hh][c][1]);
+            }
           }
         }
       }
@@ -523,21 +586,26 @@ torch::Tensor qk_prepare_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_
   }
   auto q = torch::empty({T, H, mp != nullptr ? (int64_t)G * dk : (int64_t)dk}, proj.options());
   if (T == 0) return q;
-  const size_t lds = (size_t)(H + G) * dk * sizeof(float);
+  const size_t lds = ((size_t)(H + G) * dk + 2 * half + (mp != nullptr ? H * H : 0)) * sizeof(float);
   TORCH_CHECK(lds <= 64 * 1024, "qk_prepare_kv_write: heads * dim too large");
+  TORCH_CHECK(half <= 256, "qk_prepare_kv_write: more than 512 rotated entries");
   auto stream = at::cuda::getCurrentCUDAStream();
-  if (proj.scalar_type() == at::kBFloat16)
-    qk_prepare_kv_write_kernel<bf16_t><<<T, 256, lds, stream>>>(
-        reinterpret_cast<const bf16_t*>(proj.data_ptr()), proj.stride(0), H, G, dk, vd, qw, kw,
-        (float)eps, positions.data_ptr<int>(), fp, half, (float)mag, mp, page_slot.data_ptr<int>(),
-        reinterpret_cast<bf16_t*>(cache.data_ptr()), reinterpret_cast<bf16_t*>(q.data_ptr()));
-  else {
-    SM_CHECK_F32(proj);
-    qk_prepare_kv_write_kernel<float><<<T, 256, lds, stream>>>(
-        proj.data_ptr<float>(), proj.stride(0), H, G, dk, vd, qw, kw, (float)eps,
-        positions.data_ptr<int>(), fp, half, (float)mag, mp, page_slot.data_ptr<int>(),
-        cache.data_ptr<float>(), q.data_ptr<float>());
-  }
+  const bool is_bf16 = proj.scalar_type() == at::kBFloat16;
+  if (!is_bf16) SM_CHECK_F32(proj);
+  // outputs two at a time: even sizes, rows that start on 4-byte (bf16) or
+  // 8-byte (fp32) borders
+  const int64_t esz = is_bf16 ? 2 : 4;
+  const bool pair = dk % 2 == 0 && vd % 2 == 0 && proj.stride(0) % 2 == 0 &&
+                    reinterpret_cast<uintptr_t>(proj.data_ptr()) % (2 * esz) == 0;
+#define QKP_LAUNCH(TY, PAIRV)                                                                  \
+  qk_prepare_kv_write_kernel<TY, PAIRV><<<T, 256, lds, stream>>>(                              \
+      reinterpret_cast<const TY*>(proj.data_ptr()), proj.stride(0), H, G, dk, vd, qw, kw,      \
+      (float)eps, positions.data_ptr<int>(), fp, half, (float)mag, mp,                         \
+      page_slot.data_ptr<int>(), reinterpret_cast<TY*>(cache.data_ptr()),                      \
+      reinterpret_cast<TY*>(q.data_ptr()))
+  if (is_bf16) { if (pair) QKP_LAUNCH(bf16_t, true); else QKP_LAUNCH(bf16_t, false); }
+  else { if (pair) QKP_LAUNCH(float, true); else QKP_LAUNCH(float, false); }
+#undef QKP_LAUNCH
   SM_CHECK_LAUNCH();
   return q;
 }

@@ -5,13 +5,18 @@
 // their online softmax and their value sums. The keys a tile can see are one
 // list: the kept first tokens that lie before the window of the tile's first
 // query, then everything from that window's start to the tile's last query;
-// the list is walked in blocks of 64 keys whose key columns (the head's kv
-// head, or the whole key row for folded queries) and V rows (transposed) are
-// staged in LDS once per tile.
+// the list is walked in blocks of KB keys (64; 32 for the wide key rows of
+// folded queries, so that more than one workgroup fits a CU) whose key columns
+// (the head's kv head, or the whole key row for folded queries) and V rows
+// (transposed) are staged in LDS once per tile.
 //   scores   MFMA 16x16x32: A = the wave's queries (registers, loaded once),
 //            B = K rows from LDS
 //   softmax  fp32 in the MFMA's result layout; distance bias and mask per
-//            score; row reductions over the 16 lanes of a row
+//            score; row reductions over the 16 lanes of a row by lane
+//            permutes. The distance bias depends on (head, distance) only and
+//            a wave's 16 queries meet a block's keys at KB + 15 distances:
+//            the wave tabulates those once per block instead of taking a
+//            logarithm per score
 //   values   the fp32 weights go through a wave-private LDS tile to the A
 //            layout and are split into two bf16 terms (p = hi + lo, error
 //            <= 2^-17 p); B = V^T from LDS; fp32 accumulation
@@ -25,13 +30,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 namespace {
 
-#define WAM_KB 64          // keys per block
-#define WAM_VP 72          // v_lds row pitch (bf16): 64 keys + 8
-#define WAM_PP 68          // p_lds row pitch (floats): 64 keys + 4
-
 // NT: 16-column value tiles per wave (vd <= 16 NT); KS: 32-entry steps of the
-// query/key dot product held in registers (KD <= 32 KS).
-template <int NT, int KS>
+// query/key dot product held in registers (KD <= 32 KS); KB: keys per block;
+// DIST: the distance bias is taken off the scores (r1, r2 given).
+template <int NT, int KS, int KB, bool DIST>
 __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
     const bf16_t* __restrict__ q, int KD,  // [Tn, H, KD]
     const bf16_t* __restrict__ cache,      // [rows, G (dk + vd)]
@@ -46,10 +48,15 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   const int ksteps = (KD + 31) / 32;
   const int KP = ksteps * 32 + 8;                  // k_lds row pitch (bf16)
   const int NVp = (vd + 15) / 16 * 16;
-  bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem);                 // [64][KP]
+  constexpr int WAM_KB = KB;
+  constexpr int WAM_VP = KB + 8;                   // v_lds row pitch (bf16)
+  constexpr int WAM_PP = KB + 4;                   // p_lds row pitch (floats)
+  constexpr int WAM_TB = KB + 16;                  // distance-bias table per wave
+  bf16_t* k_lds = reinterpret_cast<bf16_t*>(smem);                 // [KB][KP]
   bf16_t* v_lds = k_lds + WAM_KB * KP;                             // [NVp][WAM_VP]
   float* p_all = reinterpret_cast<float*>(v_lds + NVp * WAM_VP);   // [4][16][WAM_PP]
-  int* krow = reinterpret_cast<int*>(p_all + 4 * 16 * WAM_PP);     // [64]
+  int* krow = reinterpret_cast<int*>(p_all + 4 * 16 * WAM_PP);     // [KB]
+  float* tb_all = reinterpret_cast<float*>(krow + KB);             // [4][WAM_TB], DIST only
 
   const int tile = blockIdx.x, hd = blockIdx.y;
   const int b = tiles[3 * tile], t0 = tiles[3 * tile + 1], nq = tiles[3 * tile + 2];
@@ -65,8 +72,9 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   const int nblk = (n + WAM_KB - 1) / WAM_KB;
   const int* bt = block_tables + (int64_t)b * max_nb;
   float* p_lds = p_all + wave * 16 * WAM_PP;
+  float* tb = tb_all + wave * WAM_TB;
   const bool active = wave * 16 < nq;
-  const float a1 = (r1 != nullptr) ? r1[hd] : 0.f, a2 = (r1 != nullptr) ? r2[hd] : 0.f;
+  const float a1 = DIST ? r1[hd] : 0.f, a2 = DIST ? r2[hd] : 0.f;
 
   // the wave's queries as A fragments: row lrow, k = ks * 32 + lk * 8 ..
   bf16v8 qf[KS];
@@ -131,9 +139,21 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
       if (window > 0 && jb0 + WAM_KB - 1 < wq_first - window + 1 && jb0 >= keep) continue;
     }
 
-    f32x4 s[4];
+    // distance bias of this wave and block: the block's keys are consecutive
+    // positions jb0 .. jb0 + KB - 1 once the list is past the kept tokens, and
+    // tb[(query - 16 wave) + (KB - 1 - key column)] covers every pair
+    const bool tabled = DIST && i0 >= nf;
+    if (DIST && tabled) {
+      const int dbase = p0 + wave * 16 - (lo + (i0 - nf)) - (KB - 1);
+      for (int i = l; i < KB + 15; i += 64)
+        tb[i] = a1 * log1pf(a2 * (float)max(dbase + i, 0));
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+    }
+
+    f32x4 s[KB / 16];
     #pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
+    for (int ct = 0; ct < KB / 16; ++ct) {
       s[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
       #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -150,31 +170,32 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
     for (int r = 0; r < 4; ++r) {
       const int qi = wave * 16 + lk * 4 + r;
       const int prow = (qi < nq) ? p0 + qi : -1;
-      float sv[4];
+      float sv[KB / 16];
       float bm = -INFINITY;
       #pragma unroll
-      for (int ct = 0; ct < 4; ++ct) {
+      for (int ct = 0; ct < KB / 16; ++ct) {
         const int i = i0 + ct * 16 + lrow;
         const int j = (i < nf) ? i : lo + (i - nf);
         const bool seen = i < n && j <= prow && (window <= 0 || prow - j < window || j < keep);
         float x = s[ct][r] * scale;
-        if (r1 != nullptr && seen) x -= a1 * log1pf(a2 * (float)(prow - j));
+        if (DIST) {
+          if (tabled) x -= tb[lk * 4 + r + (KB - 1) - (ct * 16 + lrow)];
+          else if (seen) x -= a1 * log1pf(a2 * (float)(prow - j));
+        }
         sv[ct] = seen ? x : -INFINITY;
         bm = fmaxf(bm, sv[ct]);
       }
-      #pragma unroll
-      for (int off = 8; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, SM_WAVE));
+      bm = sm_row16_max(bm);
       const float mn = fmaxf(m[r], bm);
       const float c = (mn == -INFINITY) ? 1.0f : expf(m[r] - mn);
       float ps = 0.f;
       #pragma unroll
-      for (int ct = 0; ct < 4; ++ct) {
+      for (int ct = 0; ct < KB / 16; ++ct) {
         const float pv = (sv[ct] == -INFINITY) ? 0.f : expf(sv[ct] - mn);
         ps += pv;
         p_lds[(lk * 4 + r) * WAM_PP + ct * 16 + lrow] = pv;
       }
-      #pragma unroll
-      for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, SM_WAVE);
+      ps = sm_row16_sum(ps);
       lsum[r] = lsum[r] * c + ps;
       m[r] = mn;
       cr[r] = c;
@@ -182,9 +203,9 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xc07f);
     // weights as A fragments: row lrow, keys ks2 * 32 + lk * 8 ..
-    bf16v8 a_hi[2], a_lo[2];
+    bf16v8 a_hi[KB / 32], a_lo[KB / 32];
     #pragma unroll
-    for (int ks2 = 0; ks2 < 2; ++ks2) {
+    for (int ks2 = 0; ks2 < KB / 32; ++ks2) {
       const float4 w0 = *reinterpret_cast<const float4*>(p_lds + lrow * WAM_PP + ks2 * 32 + lk * 8);
       const float4 w1 = *reinterpret_cast<const float4*>(p_lds + lrow * WAM_PP + ks2 * 32 + lk * 8 + 4);
       const float pv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
@@ -202,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
         #pragma unroll
         for (int r = 0; r < 4; ++r) a[r] *= cr[r];
         #pragma unroll
-        for (int ks2 = 0; ks2 < 2; ++ks2) {
+        for (int ks2 = 0; ks2 < KB / 32; ++ks2) {
           const bf16v8 vf = *reinterpret_cast<const bf16v8*>(
               v_lds + (nt * 16 + lrow) * WAM_VP + ks2 * 32 + lk * 8);
           a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi[ks2], vf, a, 0, 0, 0);
@@ -230,9 +251,13 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   }
 }
 
-size_t wam_lds_bytes(int KD, int vd) {
+#define WAM_KEYS 32   // keys per block
+
+size_t wam_lds_bytes(int KD, int vd, bool dist) {
   const int ksteps = (KD + 31) / 32, KP = ksteps * 32 + 8, NVp = (vd + 15) / 16 * 16;
-  return (size_t)WAM_KB * KP * 2 + (size_t)NVp * WAM_VP * 2 + 4 * 16 * WAM_PP * 4 + WAM_KB * 4;
+  const int KB = WAM_KEYS;
+  return (size_t)KB * KP * 2 + (size_t)NVp * (KB + 8) * 2 + 4 * 16 * (KB + 4) * 4 + KB * 4 +
+         (dist ? 4 * (KB + 16) * 4 : 0);
 }
 
 }  // namespace
@@ -241,7 +266,7 @@ size_t wam_lds_bytes(int KD, int vd) {
 // kv_heads * dim for folded queries) and the value size are multiples of 8
 bool window_attention_mfma_fits(int KD, int vd) {
   return KD % 8 == 0 && vd % 8 == 0 && KD <= 512 && vd <= 256 &&
-         wam_lds_bytes(KD, vd) <= 150 * 1024;
+         wam_lds_bytes(KD, vd, true) <= 150 * 1024;
 }
 
 void window_attention_mfma(torch::Tensor q, int KD, torch::Tensor cache, int H, int G, int dk, int vd,
@@ -252,11 +277,11 @@ void window_attention_mfma(torch::Tensor q, int KD, torch::Tensor cache, int H, 
   const int ntiles = tiles.size(0);
   if (q.size(0) == 0 || ntiles == 0) return;
   auto stream = at::cuda::getCurrentCUDAStream();
-  const size_t lds = wam_lds_bytes(KD, vd);
+  const size_t lds = wam_lds_bytes(KD, vd, r1 != nullptr);
   dim3 grid(ntiles, H);
-#define WAM_LAUNCH(NT, KS)                                                                     \
+#define WAM_LAUNCH(NT, KS, KB, DIST)                                                           \
   do {                                                                                         \
-    auto kern = window_attention_mfma_kernel<NT, KS>;                                          \
+    auto kern = window_attention_mfma_kernel<NT, KS, KB, DIST>;                                        \
     static int raised = 0;                                                                     \
     if (lds > 64 * 1024 && (int)lds > raised) {                                                \
       TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                     \
@@ -271,15 +296,21 @@ void window_attention_mfma(torch::Tensor q, int KD, torch::Tensor cache, int H, 
         H, G, dk, vd, whole_key, scale, window, keep, r1, r2,                                  \
         reinterpret_cast<const bf16_t*>(gate), ldg, reinterpret_cast<bf16_t*>(out.data_ptr())); \
   } while (0)
-#define WAM_BY_KS(NT)                                  \
+#define WAM_BY_KS(NT, DIST)                            \
   do {                                                 \
-    if (KD <= 128) WAM_LAUNCH(NT, 4);                  \
-    else if (KD <= 256) WAM_LAUNCH(NT, 8);             \
-    else WAM_LAUNCH(NT, 16);                           \
+    if (KD <= 128) WAM_LAUNCH(NT, 4, WAM_KEYS, DIST);        \
+    else if (KD <= 256) WAM_LAUNCH(NT, 8, WAM_KEYS, DIST);   \
+    else WAM_LAUNCH(NT, 16, WAM_KEYS, DIST);                 \
   } while (0)
-  if (vd <= 64) WAM_BY_KS(4);
-  else if (vd <= 128) WAM_BY_KS(8);
-  else WAM_BY_KS(16);
+#define WAM_BY_NT(DIST)                                \
+  do {                                                 \
+    if (vd <= 64) WAM_BY_KS(4, DIST);                  \
+    else if (vd <= 128) WAM_BY_KS(8, DIST);            \
+    else WAM_BY_KS(16, DIST);                          \
+  } while (0)
+  if (r1 != nullptr) WAM_BY_NT(true);
+  else WAM_BY_NT(false);
+#undef WAM_BY_NT
 #undef WAM_BY_KS
 #undef WAM_LAUNCH
   SM_CHECK_LAUNCH();
