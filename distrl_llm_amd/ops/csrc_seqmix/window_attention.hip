@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();                 // pw and krow are rewritten next round
+    __builtin_amdgcn_wave_barrier();                 // pw and krow are rewritten for the next block
   }
   // every wave leaves (max, sum, weighted values) per head; wave 0 merges them
   // in order. A wave (or a whole share) without a block has max = -inf.
