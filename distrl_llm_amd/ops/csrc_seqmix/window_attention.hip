@@ -587,7 +587,7 @@ torch::Tensor qk_prepare_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_
   auto q = torch::empty({T, H, mp != nullptr ? (int64_t)G * dk : (int64_t)dk}, proj.options());
   if (T == 0) return q;
   const size_t lds = ((size_t)(H + G) * dk + 2 * half + (mp != nullptr ? H * H : 0)) * sizeof(float);
-  TORCH_CHECK(lds <= 64 * 1024, "qk_prepare_kv_write: heads * dim too large");
+  TORCH_CHECK(lds <= 150 * 1024, "qk_prepare_kv_write: heads * dim too large");
   TORCH_CHECK(half <= 256, "qk_prepare_kv_write: more than 512 rotated entries");
   auto stream = at::cuda::getCurrentCUDAStream();
   const bool is_bf16 = proj.scalar_type() == at::kBFloat16;
@@ -598,11 +598,21 @@ torch::Tensor qk_prepare_kv_write(torch::Tensor proj, int64_t heads, int64_t kv_
   const bool pair = dk % 2 == 0 && vd % 2 == 0 && proj.stride(0) % 2 == 0 &&
                     reinterpret_cast<uintptr_t>(proj.data_ptr()) % (2 * esz) == 0;
 #define QKP_LAUNCH(TY, PAIRV)                                                                  \
-  qk_prepare_kv_write_kernel<TY, PAIRV><<<T, 256, lds, stream>>>(                              \
-      reinterpret_cast<const TY*>(proj.data_ptr()), proj.stride(0), H, G, dk, vd, qw, kw,      \
-      (float)eps, positions.data_ptr<int>(), fp, half, (float)mag, mp,                         \
-      page_slot.data_ptr<int>(), reinterpret_cast<TY*>(cache.data_ptr()),                      \
-      reinterpret_cast<TY*>(q.data_ptr()))
+  do {                                                                                         \
+    auto kern = qk_prepare_kv_write_kernel<TY, PAIRV>;                                         \
+    static int raised = 0;     /* per variant; not repeated under graph capture */             \
+    if (lds > 64 * 1024 && (int)lds > raised) {                                                \
+      TORCH_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                     \
+                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess,     \
+                  "qk_prepare_kv_write: cannot raise the LDS limit");                          \
+      raised = (int)lds;                                                                       \
+    }                                                                                          \
+    kern<<<T, 256, lds, stream>>>(                                                             \
+        reinterpret_cast<const TY*>(proj.data_ptr()), proj.stride(0), H, G, dk, vd, qw, kw,    \
+        (float)eps, positions.data_ptr<int>(), fp, half, (float)mag, mp,                       \
+        page_slot.data_ptr<int>(), reinterpret_cast<TY*>(cache.data_ptr()),                    \
+        reinterpret_cast<TY*>(q.data_ptr()));                                                  \
+  } while (0)
   if (is_bf16) { if (pair) QKP_LAUNCH(bf16_t, true); else QKP_LAUNCH(bf16_t, false); }
   else { if (pair) QKP_LAUNCH(float, true); else QKP_LAUNCH(float, false); }
 #undef QKP_LAUNCH

@@ -39,3 +39,31 @@ def test_trace_range_propagates_exceptions():
     with pytest.raises(KeyError):
         with trace_range("x"):
             raise KeyError("boom")
+
+
+def test_collector_paused_for_captures():
+    """Garbage is collected before the block and the cyclic collector stays
+    off inside it, whatever it was before."""
+    import gc
+
+    from distrl_llm_amd.utils.capture import collector_paused
+
+    class Node:
+        pass
+
+    a, b = Node(), Node()
+    a.other, b.other = b, a
+    import weakref
+    gone = weakref.ref(a)
+    del a, b
+    assert gc.isenabled()
+    with collector_paused():
+        assert gone() is None and not gc.isenabled()
+    assert gc.isenabled()
+    gc.disable()
+    try:
+        with collector_paused():
+            assert not gc.isenabled()
+        assert not gc.isenabled()
+    finally:
+        gc.enable()
